@@ -1,0 +1,30 @@
+"""Argument checks with the reference's error convention
+(exact/exact/cpp_extension/ext_common.h:2-27): RuntimeError with the same
+message for non-device, non-contiguous, wrong-rank or wrong-dtype tensors.
+The reference also admits float16; this library computes in fp32 only."""
+import torch
+
+
+def _fail(msg):
+    raise RuntimeError(msg)
+
+
+def check_device_tensor(t, name, dim=None, dtypes=(torch.float32,)):
+    if not isinstance(t, torch.Tensor):
+        _fail(f"{name} must be a tensor!")
+    if not t.is_cuda:
+        _fail(f"{name} must be a CUDA tensor!")
+    if not t.is_contiguous():
+        _fail(f"{name} must be contiguous!")
+    if dim is not None and t.dim() != dim:
+        _fail(f"The dimension of {name} is not correct!")
+    if t.dtype not in dtypes:
+        _fail(f"The type of {name} is not correct!")
+
+
+def stream_ptr(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def ptr(t):
+    return 0 if t is None else t.data_ptr()

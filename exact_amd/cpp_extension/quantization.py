@@ -1,0 +1,200 @@
+"""Stand-in for the reference's `exact.cpp_extension.quantization` module
+(quantization.cc:137-143): pack_single_precision, unpack_single_precision,
+act_quantized_relu, act_quantized_dropout -- same names, argument order and
+error behaviour -- plus the fused entry points this library adds.
+
+Everything here is host glue: argument checks, output allocation with torch,
+and one call into libexact_hip.so on the current stream.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ..conf import config
+from ..rng import next_philox
+from ._checks import check_device_tensor, ptr, stream_ptr
+
+
+def packed_nbytes(N: int, G: int, bits: int) -> int:
+    return int(_lib.lib().exact_packed_nbytes(N, G, bits))
+
+
+def _check_bits(bits):
+    if not isinstance(bits, int) or bits <= 0 or 8 % bits != 0:
+        # TORCH_CHECK(8 % bits == 0), quantization_cuda_kernel.cu:108,198
+        raise RuntimeError("Expected 8 % bits == 0 to be true, but got false.")
+
+
+def _noise_for(shape, device):
+    """(noise tensor or None, seed, offset)."""
+    if config.noise_source is not None:
+        noise = config.noise_source(tuple(shape), device)
+        check_device_tensor(noise, "noise")
+        if noise.numel() != int(torch.Size(shape).numel()):
+            raise RuntimeError("noise has the wrong number of elements")
+        return noise, 0, 0
+    seed, offset = next_philox(device)
+    return None, seed, offset
+
+
+def pack_single_precision(data, min, max, scale, bits, stochastic):  # noqa: A002
+    """quantization.cc:37-48.  `max` is accepted and checked but, as in the
+    reference kernel, not used by the arithmetic."""
+    check_device_tensor(data, "data", 2)
+    check_device_tensor(min, "min", 1)
+    check_device_tensor(max, "max", 1)
+    check_device_tensor(scale, "scale", 1)
+    _check_bits(bits)
+    if not stochastic:
+        # TORCH_CHECK(stochastic), quantization_cuda_kernel.cu:123
+        raise RuntimeError("Expected stochastic to be true, but got false.")
+    N, G = data.shape
+    if min.numel() != N or scale.numel() != N:
+        raise RuntimeError("min / scale must have one entry per row of data")
+    packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=data.device)
+    noise, seed, offset = _noise_for(data.shape, data.device)
+    rc = _lib.lib().exact_pack_f32(ptr(data), ptr(min), ptr(scale), ptr(noise), seed, offset,
+                                   N, G, bits, ptr(packed), stream_ptr(data))
+    _lib.check(rc, "pack_single_precision")
+    return packed
+
+
+def unpack_single_precision(data, bits, scale, min, N, group_size):  # noqa: A002
+    """quantization.cc:50-62."""
+    check_device_tensor(data, "data", 1, (torch.int8,))
+    check_device_tensor(scale, "scale", 1)
+    check_device_tensor(min, "min", 1)
+    _check_bits(bits)
+    N, G = int(N), int(group_size)
+    if data.numel() < packed_nbytes(N, G, bits) - 1 or scale.numel() < N or min.numel() < N:
+        raise RuntimeError("packed data / scale / min are too short for N x group_size")
+    out = torch.empty((N, G), dtype=scale.dtype, device=data.device)
+    rc = _lib.lib().exact_unpack_f32(ptr(data), bits, ptr(scale), ptr(min), N, G, ptr(out), stream_ptr(data))
+    _lib.check(rc, "unpack_single_precision")
+    return out
+
+
+# ---- fused forms (no counterpart module function in the reference) ----------
+def minmax_pack(data, bits, want_fp32=False):
+    """One pass over data[N, G]: per-row min and scale (ops.py:39, 61-66),
+    quantise + pack, and the bf16 copies of scale / min (ops.py:80-81).
+    -> (packed int8, scale bf16, min bf16[, scale fp32, min fp32])."""
+    check_device_tensor(data, "data", 2)
+    _check_bits(bits)
+    N, G = data.shape
+    dev = data.device
+    packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=dev)
+    scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    need32 = want_fp32 or G > 1024
+    scale32 = torch.empty(N, dtype=torch.float32, device=dev) if need32 else None
+    min32 = torch.empty(N, dtype=torch.float32, device=dev) if need32 else None
+    noise, seed, offset = _noise_for(data.shape, dev)
+    rc = _lib.lib().exact_minmax_pack_f32(ptr(data), ptr(noise), seed, offset, N, G, bits, ptr(packed),
+                                          ptr(scale32), ptr(min32), ptr(scale_bf), ptr(min_bf),
+                                          stream_ptr(data))
+    _lib.check(rc, "minmax_pack")
+    if want_fp32:
+        return packed, scale_bf, min_bf, scale32, min32
+    return packed, scale_bf, min_bf
+
+
+def unpack_bf16param(data, bits, scale_bf16, min_bf16, N, group_size):
+    """unpack_single_precision with the bf16 -> fp32 widening of
+    dequantize_activation (ops.py:92-96) folded into the kernel."""
+    check_device_tensor(data, "data", 1, (torch.int8,))
+    check_device_tensor(scale_bf16, "scale", 1, (torch.bfloat16,))
+    check_device_tensor(min_bf16, "min", 1, (torch.bfloat16,))
+    _check_bits(bits)
+    N, G = int(N), int(group_size)
+    if data.numel() < packed_nbytes(N, G, bits) - 1 or scale_bf16.numel() < N or min_bf16.numel() < N:
+        raise RuntimeError("packed data / scale / min are too short for N x group_size")
+    out = torch.empty((N, G), dtype=torch.float32, device=data.device)
+    rc = _lib.lib().exact_unpack_bf16param_f32(ptr(data), bits, ptr(scale_bf16), ptr(min_bf16), N, G,
+                                               ptr(out), stream_ptr(data))
+    _lib.check(rc, "unpack_bf16param")
+    return out
+
+
+def row_minmax(data):
+    check_device_tensor(data, "data", 2)
+    N, G = data.shape
+    mn = torch.empty(N, dtype=torch.float32, device=data.device)
+    mx = torch.empty(N, dtype=torch.float32, device=data.device)
+    rc = _lib.lib().exact_row_minmax_f32(ptr(data), N, G, ptr(mn), ptr(mx), stream_ptr(data))
+    _lib.check(rc, "row_minmax")
+    return mn, mx
+
+
+# ---- 1-bit-mask activations --------------------------------------------------
+def mask_nwords(n: int) -> int:
+    return (n + 31) // 32
+
+
+class ActQuantizedReLU(torch.autograd.Function):
+    """quantization.cc:66-79: the only tensor kept for backward is the mask."""
+
+    @staticmethod
+    def forward(ctx, input):  # noqa: A002
+        n = input.numel()
+        out = torch.empty_like(input)
+        mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
+        rc = _lib.lib().exact_relu_fwd_f32(ptr(input), n, ptr(out), ptr(mask), stream_ptr(input))
+        _lib.check(rc, "act_quantized_relu")
+        ctx.save_for_backward(mask)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (mask,) = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        grad_input = torch.empty_like(grad_output)
+        rc = _lib.lib().exact_relu_bwd_f32(ptr(grad_output), ptr(mask), grad_output.numel(),
+                                           ptr(grad_input), stream_ptr(grad_output))
+        _lib.check(rc, "act_quantized_relu backward")
+        return grad_input
+
+
+def act_quantized_relu(input):  # noqa: A002
+    """quantization.cc:81-84."""
+    check_device_tensor(input, "input")
+    return ActQuantizedReLU.apply(input)
+
+
+class ActQuantizedDropout(torch.autograd.Function):
+    """quantization.cc:111-129."""
+
+    @staticmethod
+    def forward(ctx, input, p, train):  # noqa: A002
+        if not train:
+            return input
+        n = input.numel()
+        out = torch.empty_like(input)
+        mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
+        noise, seed, offset = _noise_for(input.shape, input.device)
+        rc = _lib.lib().exact_dropout_fwd_f32(ptr(input), ptr(noise), seed, offset, float(p), n,
+                                              ptr(out), ptr(mask), stream_ptr(input))
+        _lib.check(rc, "act_quantized_dropout")
+        ctx.save_for_backward(mask)
+        ctx.p = float(p)
+        ctx.train = True
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        if not getattr(ctx, "train", False):
+            return grad_output, None, None
+        (mask,) = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        grad_input = torch.empty_like(grad_output)
+        rc = _lib.lib().exact_dropout_bwd_f32(ptr(grad_output), ptr(mask), ctx.p, grad_output.numel(),
+                                              ptr(grad_input), stream_ptr(grad_output))
+        _lib.check(rc, "act_quantized_dropout backward")
+        return grad_input, None, None
+
+
+def act_quantized_dropout(input, p, train):  # noqa: A002
+    """quantization.cc:131-134."""
+    check_device_tensor(input, "input")
+    return ActQuantizedDropout.apply(input, p, train)

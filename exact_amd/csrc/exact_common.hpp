@@ -1,0 +1,99 @@
+// Shared device helpers for libexact_hip (gfx950 only, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/exact_hip.h"
+
+namespace exact {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;  // 4 wavefronts per workgroup
+
+// ---- streaming (non-temporal) 16-byte accesses -----------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4 nt_load4(const float* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+}
+__device__ __forceinline__ void nt_store4(float* p, float a, float b, float c, float d) {
+  f32x4 v = {a, b, c, d};
+  __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(p));
+}
+
+// ---- launch helpers --------------------------------------------------------
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? EXACT_OK : static_cast<int>(e);
+}
+
+// ---- Philox4x32-10 ---------------------------------------------------------
+// Block function of Salmon et al. (SC'11); the reference draws from cuRAND's
+// Philox4_32_10 (quantization_cuda_kernel.cu:77-79, 452-453).  The key is
+// wave-uniform, so its schedule lives in scalar registers.
+struct Philox4 {
+  uint32_t x, y, z, w;
+};
+
+__device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2,
+                                                 uint32_t c3, uint32_t k0, uint32_t k1) {
+  constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+  constexpr uint32_t W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = static_cast<uint64_t>(M0) * c0;
+    const uint64_t p1 = static_cast<uint64_t>(M1) * c2;
+    const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1;
+    c1 = static_cast<uint32_t>(p1);
+    c3 = static_cast<uint32_t>(p0);
+    c0 = n0;
+    c2 = n2;
+    k0 += W0;
+    k1 += W1;
+  }
+  return Philox4{c0, c1, c2, c3};
+}
+
+// 16 random bits -> uniform on (0,1): (h + 0.5) * 2^-16, exact in fp32.
+__device__ __forceinline__ float u16_to_uniform(uint32_t h) {
+  return __fmaf_rn(static_cast<float>(h), 0x1p-16f, 0x1p-17f);
+}
+
+// Eight uniforms from one Philox block: word w gives elements 2w (low half)
+// and 2w+1 (high half).
+__device__ __forceinline__ void philox_uniform8(const Philox4& r, float (&u)[8]) {
+  u[0] = u16_to_uniform(r.x & 0xFFFFu);
+  u[1] = u16_to_uniform(r.x >> 16);
+  u[2] = u16_to_uniform(r.y & 0xFFFFu);
+  u[3] = u16_to_uniform(r.y >> 16);
+  u[4] = u16_to_uniform(r.z & 0xFFFFu);
+  u[5] = u16_to_uniform(r.z >> 16);
+  u[6] = u16_to_uniform(r.w & 0xFFFFu);
+  u[7] = u16_to_uniform(r.w >> 16);
+}
+
+// ---- bf16 ------------------------------------------------------------------
+// fp32 -> bf16 bits, round to nearest even (what Tensor.to(torch.bfloat16)
+// does at ops.py:80-81 of the reference).
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t b = __float_as_uint(f);
+  if ((b & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((b >> 16) & 0x8000u) | 0x7FC0u;
+  b += 0x7FFFu + ((b >> 16) & 1u);
+  return static_cast<uint16_t>(b >> 16);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return __uint_as_float(static_cast<uint32_t>(h) << 16);
+}
+
+// ---- cross-lane ------------------------------------------------------------
+// Butterfly min / max over aligned groups of `span` lanes (span a power of two
+// <= 64).  Every lane of the group ends with the group's result.
+__device__ __forceinline__ void group_minmax(float& mn, float& mx, int span) {
+  for (int m = 1; m < span; m <<= 1) {
+    mn = fminf(mn, __shfl_xor(mn, m));
+    mx = fmaxf(mx, __shfl_xor(mx, m));
+  }
+}
+
+}  // namespace exact

@@ -1,0 +1,549 @@
+// Per-row min/range, stochastic-rounding quantise + bit-pack, and the matching
+// unpack + dequantise, for [N, G] fp32 activations on gfx950.
+//
+// Algorithm restated from the reference kernels
+//   pack_single_precision_kernel    quantization_cuda_kernel.cu:63-94
+//   unpack_single_precision_kernel  quantization_cuda_kernel.cu:158-185
+// and the torch glue around them (ops.py:20-98, qsheme.py:41-48); the
+// decomposition below is this library's own.
+//
+// Work unit: an "oct" = 8 consecutive columns of one row (32 B of fp32, one
+// Philox block of noise, 8 quantised bytes before bit-packing).  A row is
+// owned by `lpr` adjacent lanes (a power of two <= 32, so a row never leaves
+// its wavefront) with OPT octs per lane; a 256-thread workgroup owns
+// 256 / lpr consecutive rows (always a multiple of 8, so it owns whole
+// row-groups of every bit width).  Row min/max are butterfly reductions in
+// registers; the quantised bytes are staged in LDS, where the lane that owns
+// the first row of a group ORs the 8/bits rows of that group together and
+// writes the packed bytes with one vector store.
+//
+// All arithmetic that decides a quantised value is written as separate fp32
+// operations and this file is compiled with -ffp-contract=off, so the result
+// is the unfused expression of the reference source.
+
+#include "exact_common.hpp"
+
+namespace exact {
+
+// ---------------------------------------------------------------------------
+// loads / stores of one oct with `nv` (0..8) valid leading elements
+// ---------------------------------------------------------------------------
+template <int VEC, bool FULL>
+__device__ __forceinline__ void load_oct(const float* __restrict__ p, int nv, float (&v)[8]) {
+  if constexpr (VEC == 4) {
+    f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = a;
+    if (FULL || nv > 0) a = nt_load4(p);
+    if (FULL || nv > 4) b = nt_load4(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (i < nv) ? __builtin_nontemporal_load(p + i) : 0.f;
+  }
+}
+
+template <int VEC, bool FULL>
+__device__ __forceinline__ void store_oct(float* __restrict__ p, int nv, const float (&v)[8]) {
+  if constexpr (VEC == 4) {
+    if (FULL || nv > 0) nt_store4(p, v[0], v[1], v[2], v[3]);
+    if (FULL || nv > 4) nt_store4(p + 4, v[4], v[5], v[6], v[7]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < nv) __builtin_nontemporal_store(v[i], p + i);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// pack
+// ---------------------------------------------------------------------------
+struct PackArgs {
+  const float* x;
+  const float* noise;     // nullable
+  const float* mn_in;     // two-step form only
+  const float* scale_in;  // two-step form only
+  uint32_t seed_lo, seed_hi, off_lo, off_hi;
+  int64_t N;
+  int G;
+  int opr;        // octs per row
+  int lpr_log2;   // log2(lanes per row)
+  int out_vec;    // 8, 4 or 1: widest aligned store of packed bytes
+  uint8_t* packed;
+  int64_t pad_index;  // index of the trailing pad byte
+  float* scale_f32;
+  float* min_f32;
+  uint16_t* scale_bf16;
+  uint16_t* min_bf16;
+};
+
+template <int BITS, int OPT, int VEC, bool FULL, bool NOISE_IN, bool FUSED>
+__global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
+  constexpr int WPT = 8 / BITS;
+  constexpr float B = static_cast<float>((1 << BITS) - 1);
+  __shared__ uint2 stage[OPT * kBlock];
+
+  const int t = threadIdx.x;
+  const int lpr = 1 << a.lpr_log2;
+  const int lane_in_row = t & (lpr - 1);
+  const int row_local = t >> a.lpr_log2;
+  const int rows_per_wg = kBlock >> a.lpr_log2;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * rows_per_wg + row_local;
+  const bool row_ok = n < a.N;
+  const int oct_base = blockIdx.y * (lpr * OPT);  // 0 in the fused form
+  const int64_t row_off = n * a.G;
+
+  float v[OPT][8];
+  int nv[OPT];
+#pragma unroll
+  for (int k = 0; k < OPT; ++k) {
+    const int j = oct_base + lane_in_row + k * lpr;
+    const int d0 = 8 * j;
+    nv[k] = (row_ok && j < a.opr) ? min(8, a.G - d0) : 0;
+    if (FULL && !row_ok) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[k][i] = 0.f;
+    } else {
+      load_oct<VEC, FULL>(a.x + row_off + d0, nv[k], v[k]);
+    }
+  }
+
+  float mnv = 0.f, sc = 0.f;
+  if constexpr (FUSED) {
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (FULL || i < nv[k]) {
+          lo = fminf(lo, v[k][i]);
+          hi = fmaxf(hi, v[k][i]);
+        }
+      }
+    }
+    group_minmax(lo, hi, lpr);
+    mnv = lo;
+    sc = B / (hi - lo);  // ops.py:39, fp32 division
+    if (row_ok && lane_in_row == 0) {
+      if (a.scale_f32) a.scale_f32[n] = sc;
+      if (a.min_f32) a.min_f32[n] = mnv;
+      if (a.scale_bf16) a.scale_bf16[n] = f32_to_bf16_rne(sc);
+      if (a.min_bf16) a.min_bf16[n] = f32_to_bf16_rne(mnv);
+    }
+  } else {
+    if (row_ok) {
+      mnv = a.mn_in[n];
+      sc = a.scale_in[n];
+    }
+  }
+
+#pragma unroll
+  for (int k = 0; k < OPT; ++k) {
+    const int j = oct_base + lane_in_row + k * lpr;
+    float u[8];
+    if constexpr (NOISE_IN) {
+      if (FULL && !row_ok) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u[i] = 0.f;
+      } else {
+        load_oct<VEC, FULL>(a.noise + row_off + 8 * j, nv[k], u);
+      }
+    } else {
+      const Philox4 r = philox4x32_10(static_cast<uint32_t>(j), static_cast<uint32_t>(n),
+                                      a.off_lo, a.off_hi, a.seed_lo, a.seed_hi);
+      philox_uniform8(r, u);
+    }
+    uint32_t q[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // quantization_cuda_kernel.cu:89, one rounding per operation
+      float tq = v[k][i] - mnv;
+      tq = tq * sc;
+      tq = tq + u[i];
+      tq = tq - 0.5f;
+      tq = fmaxf(tq, 0.f);
+      const uint32_t qi = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
+      q[i] = ((FULL ? row_ok : (i < nv[k])) ? qi : 0u) & 0xFFu;
+    }
+    stage[k * kBlock + t] = make_uint2(q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24),
+                                       q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24));
+  }
+  __syncthreads();
+
+  // The lane holding the first row of a row-group packs the whole group.
+  if ((row_local & (WPT - 1)) == 0 && row_ok) {
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) {
+      const int j = oct_base + lane_in_row + k * lpr;
+      if (j >= a.opr) continue;
+      uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+      for (int i = 0; i < WPT; ++i) {
+        // uint8 accumulator of the reference: bits shifted past bit 7 vanish
+        constexpr uint32_t kByte = 0x01010101u;
+        const uint32_t keep = (0xFFu >> (i * BITS)) * kByte;
+        const uint2 s = stage[k * kBlock + t + i * lpr];
+        w0 |= (s.x & keep) << (i * BITS);
+        w1 |= (s.y & keep) << (i * BITS);
+      }
+      const int d0 = 8 * j;
+      uint8_t* dst = a.packed + (n / WPT) * a.G + d0;
+      if (a.out_vec == 8) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(w0, w1);
+      } else if (a.out_vec == 4) {
+        *reinterpret_cast<uint32_t*>(dst) = w0;
+        if (d0 + 4 < a.G) *reinterpret_cast<uint32_t*>(dst + 4) = w1;
+      } else {
+        const int cnt = min(8, a.G - d0);
+        for (int i = 0; i < cnt; ++i)
+          dst[i] = static_cast<uint8_t>((i < 4 ? w0 >> (8 * i) : w1 >> (8 * (i - 4))) & 0xFFu);
+      }
+    }
+  }
+  if (blockIdx.x == 0 && blockIdx.y == 0 && t == 0) a.packed[a.pad_index] = 0;
+}
+
+// ---------------------------------------------------------------------------
+// row statistics for rows longer than the fused kernel holds in registers,
+// and the stand-alone a1 entry point: one wavefront per row.
+// ---------------------------------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void row_minmax_kernel(const float* __restrict__ x, int64_t N,
+                                                            int64_t G, float* __restrict__ mn_out,
+                                                            float* __restrict__ mx_out, int bits,
+                                                            float* __restrict__ scale_f32,
+                                                            uint16_t* __restrict__ scale_bf16,
+                                                            uint16_t* __restrict__ min_bf16) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const float* row = x + n * G;
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  if constexpr (VEC == 4) {
+    const float4* r4 = reinterpret_cast<const float4*>(row);
+    for (int64_t c = lane; c < G / 4; c += kWave) {
+      const float4 q = r4[c];
+      lo = fminf(fminf(lo, q.x), fminf(q.y, fminf(q.z, q.w)));
+      hi = fmaxf(fmaxf(hi, q.x), fmaxf(q.y, fmaxf(q.z, q.w)));
+    }
+  } else {
+    for (int64_t c = lane; c < G; c += kWave) {
+      lo = fminf(lo, row[c]);
+      hi = fmaxf(hi, row[c]);
+    }
+  }
+  group_minmax(lo, hi, kWave);
+  if (lane == 0) {
+    if (mn_out) mn_out[n] = lo;
+    if (mx_out) mx_out[n] = hi;
+    if (bits > 0) {
+      const float sc = static_cast<float>((1 << bits) - 1) / (hi - lo);
+      if (scale_f32) scale_f32[n] = sc;
+      if (scale_bf16) scale_bf16[n] = f32_to_bf16_rne(sc);
+      if (min_bf16) min_bf16[n] = f32_to_bf16_rne(lo);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// unpack
+// ---------------------------------------------------------------------------
+struct UnpackArgs {
+  const uint8_t* packed;
+  const void* scale;  // float* or bf16 bits
+  const void* mn;
+  int64_t N;
+  int G;
+  int opr;
+  int lpr_log2;
+  int in_vec;  // 8, 4 or 1: widest aligned load of packed bytes
+  float* out;
+};
+
+template <int BITS, int OPT, int VEC, bool FULL, bool BF16P>
+__global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
+  constexpr int WPT = 8 / BITS;
+  constexpr uint32_t FIELD = ((1u << BITS) - 1u) * 0x01010101u;
+  const int t = threadIdx.x;
+  const int lpr = 1 << a.lpr_log2;
+  const int lane_in_row = t & (lpr - 1);
+  const int rows_per_wg = kBlock >> a.lpr_log2;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (t >> a.lpr_log2);
+  if (n >= a.N) return;
+  const int oct_base = blockIdx.y * (lpr * OPT);
+
+  float sc, mnv;
+  if constexpr (BF16P) {
+    sc = bf16_to_f32(static_cast<const uint16_t*>(a.scale)[n]);
+    mnv = bf16_to_f32(static_cast<const uint16_t*>(a.mn)[n]);
+  } else {
+    sc = static_cast<const float*>(a.scale)[n];
+    mnv = static_cast<const float*>(a.mn)[n];
+  }
+  const int shift = static_cast<int>(n & (WPT - 1)) * BITS;
+  const uint8_t* grp = a.packed + (n / WPT) * a.G;
+  float* orow = a.out + n * a.G;
+
+#pragma unroll
+  for (int k = 0; k < OPT; ++k) {
+    const int j = oct_base + lane_in_row + k * lpr;
+    if (!FULL && j >= a.opr) continue;
+    const int d0 = 8 * j;
+    const int nv = FULL ? 8 : min(8, a.G - d0);
+    uint32_t w0 = 0, w1 = 0;
+    if (FULL || a.in_vec == 8) {
+      const uint2 w = *reinterpret_cast<const uint2*>(grp + d0);
+      w0 = w.x;
+      w1 = w.y;
+    } else if (a.in_vec == 4) {
+      w0 = *reinterpret_cast<const uint32_t*>(grp + d0);
+      if (nv > 4) w1 = *reinterpret_cast<const uint32_t*>(grp + d0 + 4);
+    } else {
+      for (int i = 0; i < nv; ++i) {
+        const uint32_t byte = grp[d0 + i];
+        if (i < 4) w0 |= byte << (8 * i); else w1 |= byte << (8 * (i - 4));
+      }
+    }
+    w0 = (w0 >> shift) & FIELD;
+    w1 = (w1 >> shift) & FIELD;
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t qi = ((i < 4 ? w0 >> (8 * i) : w1 >> (8 * (i - 4))) & 0xFFu);
+      // quantization_cuda_kernel.cu:182: true division, then add
+      const float qf = static_cast<float>(qi) / sc;
+      r[i] = qf + mnv;
+    }
+    store_oct<VEC, FULL>(orow + d0, nv, r);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct Geometry {
+  int opr, lpr_log2, opt, grid_y;
+  bool full;
+};
+
+// Octs per thread and lanes per row for rows of G columns.  `max_opt` octs fit
+// in registers; longer rows are tiled over grid.y (two-step form only).
+static Geometry plan_rows(int64_t G, int max_opt) {
+  Geometry g;
+  g.opr = static_cast<int>((G + 7) / 8);
+  int opt = (g.opr + 31) / 32;
+  if (opt > max_opt) opt = max_opt;
+  if (opt == 3) opt = 4;
+  if (opt < 1) opt = 1;
+  const int lanes_needed = (g.opr + opt - 1) / opt;
+  int l2 = 0;
+  while ((1 << l2) < lanes_needed && l2 < 5) ++l2;
+  g.lpr_log2 = l2;
+  g.opt = opt;
+  const int octs_per_pass = (1 << l2) * opt;
+  g.grid_y = (g.opr + octs_per_pass - 1) / octs_per_pass;
+  g.full = (G % 8 == 0) && (g.opr == octs_per_pass * g.grid_y);
+  return g;
+}
+
+__global__ void zero_byte_kernel(uint8_t* p) { *p = 0; }
+
+static bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+template <int BITS, int OPT, bool NOISE_IN, bool FUSED>
+static void launch_pack_variant(const PackArgs& a, bool vec4, bool full, dim3 grid, hipStream_t s) {
+  if (vec4 && full)
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, true, NOISE_IN, FUSED>), grid, dim3(kBlock), 0, s, a);
+  else if (vec4)
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, false, NOISE_IN, FUSED>), grid, dim3(kBlock), 0, s, a);
+  else
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 1, false, NOISE_IN, FUSED>), grid, dim3(kBlock), 0, s, a);
+}
+
+template <int BITS, bool NOISE_IN, bool FUSED>
+static void launch_pack_opt(const PackArgs& a, int opt, bool vec4, bool full, dim3 grid, hipStream_t s) {
+  if constexpr (FUSED) {
+    if (opt == 4) return launch_pack_variant<BITS, 4, NOISE_IN, FUSED>(a, vec4, full, grid, s);
+    if (opt == 2) return launch_pack_variant<BITS, 2, NOISE_IN, FUSED>(a, vec4, full, grid, s);
+  }
+  launch_pack_variant<BITS, 1, NOISE_IN, FUSED>(a, vec4, full, grid, s);
+}
+
+template <bool NOISE_IN, bool FUSED>
+static void launch_pack_bits(const PackArgs& a, int bits, int opt, bool vec4, bool full, dim3 grid, hipStream_t s) {
+  switch (bits) {
+    case 1: return launch_pack_opt<1, NOISE_IN, FUSED>(a, opt, vec4, full, grid, s);
+    case 2: return launch_pack_opt<2, NOISE_IN, FUSED>(a, opt, vec4, full, grid, s);
+    case 4: return launch_pack_opt<4, NOISE_IN, FUSED>(a, opt, vec4, full, grid, s);
+    default: return launch_pack_opt<8, NOISE_IN, FUSED>(a, opt, vec4, full, grid, s);
+  }
+}
+
+static int check_quant_shape(int64_t N, int64_t G, int bits) {
+  if (bits != 1 && bits != 2 && bits != 4 && bits != 8) return EXACT_E_BITS;
+  if (N < 0 || G < 0 || N > 0xFFFFFFFFll || G > 0x7FFFFFF0ll) return EXACT_E_SHAPE;
+  return EXACT_OK;
+}
+
+static int pack_common(const float* x, const float* mn, const float* scale, const float* noise,
+                       uint64_t seed, uint64_t offset, int64_t N, int64_t G, int bits,
+                       uint8_t* packed, float* scale_f32, float* min_f32, uint16_t* scale_bf16,
+                       uint16_t* min_bf16, bool fused, hipStream_t s) {
+  if (int rc = check_quant_shape(N, G, bits)) return rc;
+  if (!packed) return EXACT_E_NULL;
+  const int64_t pad_index = exact_packed_nbytes(N, G, bits) - 1;
+  if (N == 0 || G == 0) {
+    // nothing but the pad byte (a kernel, not a memset node, so callers may capture it)
+    hipLaunchKernelGGL(zero_byte_kernel, dim3(1), dim3(1), 0, s, packed + pad_index);
+    return launch_status();
+  }
+  if (!x || (!fused && (!mn || !scale))) return EXACT_E_NULL;
+
+  bool do_fused = fused;
+  if (fused && G > 1024) {
+    // rows too long for registers: statistics first, then the two-step form
+    float* mn_tmp = min_f32;
+    float* sc_tmp = scale_f32;
+    if (!mn_tmp || !sc_tmp) return EXACT_E_NULL;  // caller must give fp32 outputs for G > 1024
+    const bool v4 = (G % 4 == 0) && aligned(x, 16);
+    const dim3 grid(static_cast<unsigned>((N + 3) / 4));
+    if (v4)
+      hipLaunchKernelGGL((row_minmax_kernel<4>), grid, dim3(kBlock), 0, s, x, N, G, mn_tmp,
+                         static_cast<float*>(nullptr), bits, sc_tmp, scale_bf16, min_bf16);
+    else
+      hipLaunchKernelGGL((row_minmax_kernel<1>), grid, dim3(kBlock), 0, s, x, N, G, mn_tmp,
+                         static_cast<float*>(nullptr), bits, sc_tmp, scale_bf16, min_bf16);
+    mn = mn_tmp;
+    scale = sc_tmp;
+    do_fused = false;
+  }
+
+  const Geometry g = plan_rows(G, do_fused ? 4 : 1);
+  PackArgs a;
+  a.x = x;
+  a.noise = noise;
+  a.mn_in = mn;
+  a.scale_in = scale;
+  a.seed_lo = static_cast<uint32_t>(seed);
+  a.seed_hi = static_cast<uint32_t>(seed >> 32);
+  a.off_lo = static_cast<uint32_t>(offset);
+  a.off_hi = static_cast<uint32_t>(offset >> 32);
+  a.N = N;
+  a.G = static_cast<int>(G);
+  a.opr = g.opr;
+  a.lpr_log2 = g.lpr_log2;
+  a.packed = packed;
+  a.pad_index = pad_index;
+  a.scale_f32 = do_fused ? scale_f32 : nullptr;
+  a.min_f32 = do_fused ? min_f32 : nullptr;
+  a.scale_bf16 = do_fused ? scale_bf16 : nullptr;
+  a.min_bf16 = do_fused ? min_bf16 : nullptr;
+  a.out_vec = (G % 8 == 0 && aligned(packed, 8)) ? 8 : (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
+  const bool vec4 = (G % 4 == 0) && aligned(x, 16) && (!noise || aligned(noise, 16));
+  const int rows_per_wg = kBlock >> g.lpr_log2;
+  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(g.grid_y));
+  const bool full = g.full && vec4;
+  if (do_fused) {
+    if (noise) launch_pack_bits<true, true>(a, bits, g.opt, vec4, full, grid, s);
+    else launch_pack_bits<false, true>(a, bits, g.opt, vec4, full, grid, s);
+  } else {
+    if (noise) launch_pack_bits<true, false>(a, bits, g.opt, vec4, full, grid, s);
+    else launch_pack_bits<false, false>(a, bits, g.opt, vec4, full, grid, s);
+  }
+  return launch_status();
+}
+
+template <int BITS, bool BF16P>
+static void launch_unpack_variant(const UnpackArgs& a, bool vec4, bool full, dim3 grid, hipStream_t s) {
+  if (vec4 && full)
+    hipLaunchKernelGGL((unpack_kernel<BITS, 1, 4, true, BF16P>), grid, dim3(kBlock), 0, s, a);
+  else if (vec4)
+    hipLaunchKernelGGL((unpack_kernel<BITS, 1, 4, false, BF16P>), grid, dim3(kBlock), 0, s, a);
+  else
+    hipLaunchKernelGGL((unpack_kernel<BITS, 1, 1, false, BF16P>), grid, dim3(kBlock), 0, s, a);
+}
+
+template <bool BF16P>
+static int unpack_common(const uint8_t* packed, int bits, const void* scale, const void* mn,
+                         int64_t N, int64_t G, float* out, hipStream_t s) {
+  if (int rc = check_quant_shape(N, G, bits)) return rc;
+  if (N == 0 || G == 0) return EXACT_OK;
+  if (!packed || !scale || !mn || !out) return EXACT_E_NULL;
+  const Geometry g = plan_rows(G, 1);
+  UnpackArgs a;
+  a.packed = packed;
+  a.scale = scale;
+  a.mn = mn;
+  a.N = N;
+  a.G = static_cast<int>(G);
+  a.opr = g.opr;
+  a.lpr_log2 = g.lpr_log2;
+  a.out = out;
+  a.in_vec = (G % 8 == 0 && aligned(packed, 8)) ? 8 : (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
+  const bool vec4 = (G % 4 == 0) && aligned(out, 16);
+  const bool full = g.full && vec4 && a.in_vec == 8;
+  const int rows_per_wg = kBlock >> g.lpr_log2;
+  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(g.grid_y));
+  switch (bits) {
+    case 1: launch_unpack_variant<1, BF16P>(a, vec4, full, grid, s); break;
+    case 2: launch_unpack_variant<2, BF16P>(a, vec4, full, grid, s); break;
+    case 4: launch_unpack_variant<4, BF16P>(a, vec4, full, grid, s); break;
+    default: launch_unpack_variant<8, BF16P>(a, vec4, full, grid, s); break;
+  }
+  return launch_status();
+}
+
+}  // namespace exact
+
+using namespace exact;
+
+extern "C" {
+
+int64_t exact_packed_nbytes(int64_t N, int64_t G, int bits) {
+  if (bits != 1 && bits != 2 && bits != 4 && bits != 8) return EXACT_E_BITS;
+  const int64_t wpt = 8 / bits;
+  const int64_t n_round = N + (wpt - N % wpt) % wpt;
+  return (static_cast<int64_t>(bits) * n_round * G + 8) / 8;
+}
+
+int exact_row_minmax_f32(const float* x, int64_t N, int64_t G, float* mn, float* mx, void* stream) {
+  if (N < 0 || G <= 0) return N == 0 || G == 0 ? (N < 0 || G < 0 ? EXACT_E_SHAPE : EXACT_OK) : EXACT_E_SHAPE;
+  if (N == 0) return EXACT_OK;
+  if (!x || !mn || !mx) return EXACT_E_NULL;
+  const dim3 grid(static_cast<unsigned>((N + 3) / 4));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (G % 4 == 0 && aligned(x, 16))
+    hipLaunchKernelGGL((row_minmax_kernel<4>), grid, dim3(kBlock), 0, s, x, N, G, mn, mx, 0,
+                       static_cast<float*>(nullptr), static_cast<uint16_t*>(nullptr),
+                       static_cast<uint16_t*>(nullptr));
+  else
+    hipLaunchKernelGGL((row_minmax_kernel<1>), grid, dim3(kBlock), 0, s, x, N, G, mn, mx, 0,
+                       static_cast<float*>(nullptr), static_cast<uint16_t*>(nullptr),
+                       static_cast<uint16_t*>(nullptr));
+  return launch_status();
+}
+
+int exact_pack_f32(const float* x, const float* mn, const float* scale, const float* noise,
+                   uint64_t seed, uint64_t offset, int64_t N, int64_t G, int bits, uint8_t* packed,
+                   void* stream) {
+  return pack_common(x, mn, scale, noise, seed, offset, N, G, bits, packed, nullptr, nullptr, nullptr,
+                     nullptr, false, static_cast<hipStream_t>(stream));
+}
+
+int exact_minmax_pack_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset,
+                          int64_t N, int64_t G, int bits, uint8_t* packed, float* scale_f32,
+                          float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, void* stream) {
+  return pack_common(x, nullptr, nullptr, noise, seed, offset, N, G, bits, packed, scale_f32, min_f32,
+                     scale_bf16, min_bf16, true, static_cast<hipStream_t>(stream));
+}
+
+int exact_unpack_f32(const uint8_t* packed, int bits, const float* scale, const float* mn, int64_t N,
+                     int64_t G, float* out, void* stream) {
+  return unpack_common<false>(packed, bits, scale, mn, N, G, out, static_cast<hipStream_t>(stream));
+}
+
+int exact_unpack_bf16param_f32(const uint8_t* packed, int bits, const uint16_t* scale_bf16,
+                               const uint16_t* min_bf16, int64_t N, int64_t G, float* out, void* stream) {
+  return unpack_common<true>(packed, bits, scale_bf16, min_bf16, N, G, out, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

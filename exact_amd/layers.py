@@ -1,0 +1,159 @@
+"""Drop-in quantised layers with the names, constructor arguments and
+forward signatures of exact/exact/layers.py in the reference (QLinear :268,
+QGCNConv :215, QSAGEConv :123, QBatchNorm1d :340, QReLU :284, QDropout :316,
+QDropout2 :328).  In eval mode every layer runs the stock op, as there."""
+import torch
+import torch.nn.functional as F
+from torch.nn import Parameter
+
+from .conf import config
+from .cpp_extension import quantization as ext_quantization
+from .nn import GCNConv, SAGEConv, glorot
+from .ops import input2rp, qbatch_norm, qlinear, quantize_activation
+from .qsheme import QScheme
+from .spmm import QMatmul
+
+
+class QLinear(torch.nn.Linear):
+    def __init__(self, input_features, output_features, bias=True, rp=True):
+        super().__init__(input_features, output_features, bias)
+        self.scheme = QScheme("linear") if config.single_precision else None
+        self.rp = rp
+
+    def forward(self, input, quantized=None, randmat=None):  # noqa: A002
+        if self.training:
+            return qlinear.apply(input, self.weight, self.bias, quantized, randmat, self.scheme, self.rp)
+        return super().forward(input)
+
+
+class QGCNConv(GCNConv):
+    """layers.py:215-265: the weight is stored [out, in] and the linear map is
+    a qlinear; propagation is a quantised SpMM."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.weight = Parameter(torch.Tensor(self.out_channels, self.in_channels))
+        self.msg_and_aggr_func = QMatmul(self.aggr)
+        self.lin_scheme = QScheme("linear") if config.single_precision else None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        glorot(self.weight)
+        if self.bias is not None:
+            self.bias.data.zero_()
+        self._cached_adj_t = None
+
+    def forward(self, x, edge_index, edge_weight=None):
+        adj_t = self._normalized(edge_index)
+        if self.training:
+            # layers.py:252 passes lin_scheme in the `randmat` slot; with
+            # kept_frac == 1 that slot is unused, so the numbers are those of
+            # a qlinear without a scheme.  Here the scheme is passed as scheme.
+            x = qlinear.apply(x, self.weight, None, None, None, self.lin_scheme)
+        else:
+            x = F.linear(x, self.weight, None)
+        out = self.message_and_aggregate(adj_t, x)
+        if self.bias is not None:
+            out = out + self.bias
+        return out
+
+    def message_and_aggregate(self, adj_t, x):
+        return self.msg_and_aggr_func(adj_t, x)
+
+
+class QSAGEConv(SAGEConv):
+    """layers.py:123-178: the input is projected + quantised ONCE and the same
+    compressed copy serves the mean aggregation and lin_r."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        in_channels = self.in_channels
+        if isinstance(in_channels, int):
+            in_channels = (in_channels, in_channels)
+        bias = self.lin_l.bias is not None
+        self.lin_l = QLinear(in_channels[0], self.out_channels, bias=bias, rp=True)
+        if self.root_weight:
+            self.lin_r = QLinear(in_channels[1], self.out_channels, bias=False, rp=True)
+        self.msg_and_aggr_func = QMatmul(self.aggr)
+        self.scheme = QScheme("sage") if config.single_precision else None
+        self.reset_parameters()
+
+    def forward(self, x, edge_index, size=None):
+        if isinstance(x, torch.Tensor):
+            x = (x, x)
+            l_eq_r = True
+        else:
+            l_eq_r = False
+        if l_eq_r and self.training:
+            if config.kept_frac < 1.0:
+                kept_acts = int(config.kept_frac * x[0].shape[1] + 0.999)
+                dim_reduced_input, randmat = input2rp(x[0], kept_acts)
+            else:
+                dim_reduced_input, randmat = x[0], None
+            quantized = quantize_activation(dim_reduced_input, self.scheme)
+        else:
+            quantized, randmat = None, None
+        out = self.message_and_aggregate(edge_index, x, quantized=quantized, randmat=randmat)
+        out = self.lin_l(out)
+        x_r = x[1]
+        if self.root_weight and x_r is not None:
+            out = out + self.lin_r(x_r, quantized, randmat)
+        if self.normalize:
+            out = F.normalize(out, p=2.0, dim=-1)
+        return out
+
+    def message_and_aggregate(self, adj_t, x, quantized=None, randmat=None):
+        return self.msg_and_aggr_func(adj_t, x[0], quantized=quantized, randmat=randmat)
+
+
+class QReLU(torch.nn.Module):
+    def __init__(self, inplace=False):
+        super().__init__()
+
+    def forward(self, input):  # noqa: A002
+        if self.training:
+            return ext_quantization.act_quantized_relu(input)
+        return F.relu(input)
+
+
+class QDropout(torch.nn.Module):
+    def __init__(self, p):
+        super().__init__()
+        self.p = p
+
+    def forward(self, input):  # noqa: A002
+        if self.training:
+            return ext_quantization.act_quantized_dropout(input, self.p, self.training)
+        return F.dropout(input, self.p, self.training)
+
+
+class QDropout2(torch.nn.Module):
+    def __init__(self, p):
+        super().__init__()
+        self.p = p
+
+    def forward(self, input):  # noqa: A002
+        if self.training:
+            return ext_quantization.act_quantized_dropout(input, self.p, self.training) * (1 - self.p)
+        return F.dropout(input, self.p, self.training) * (1 - self.p)
+
+
+class QBatchNorm1d(torch.nn.BatchNorm1d):
+    def __init__(self, num_features, eps=1e-05, momentum=0.1, affine=True, track_running_stats=True):
+        super().__init__(num_features, eps, momentum, affine, track_running_stats)
+        self.scheme = QScheme("batchnorm") if config.single_precision else None
+
+    def forward(self, input):  # noqa: A002
+        if not self.training:
+            return super().forward(input)
+        self._check_input_dim(input)
+        exponential_average_factor = 0.0 if self.momentum is None else self.momentum
+        if self.track_running_stats and self.num_batches_tracked is not None:
+            self.num_batches_tracked = self.num_batches_tracked + 1
+            if self.momentum is None:
+                exponential_average_factor = 1.0 / float(self.num_batches_tracked)
+        return qbatch_norm.apply(
+            input,
+            self.running_mean if self.track_running_stats else None,
+            self.running_var if self.track_running_stats else None,
+            self.weight, self.bias, True, exponential_average_factor, self.eps, self.scheme)

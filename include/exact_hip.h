@@ -1,0 +1,136 @@
+/*
+ * exact_hip.h -- C ABI of libexact_hip.so, the gfx950 (MI355X) implementation
+ * of EXACT's activation-compression and sparse-aggregation hot path.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless
+ *     stated otherwise; the caller allocates every output; the library never
+ *     allocates, frees or keeps a pointer after the call returns;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work
+ *     is enqueued on it and the call returns without synchronising;
+ *   - return value: 0 = ok, negative = argument error (EXACT_E_*), positive =
+ *     the hipError_t of a failed launch;
+ *   - re-entrant, no global state.
+ *
+ * Each declaration cites the interface of the reference extension it replaces
+ * (paths relative to exact/exact/cpp_extension/ of the reference unless they
+ * name another file).
+ */
+#ifndef EXACT_HIP_H_
+#define EXACT_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EXACT_ABI_VERSION 1
+
+#define EXACT_OK 0
+#define EXACT_E_NULL (-1)      /* a required pointer is NULL                    */
+#define EXACT_E_BITS (-2)      /* bits not in {1,2,4,8} (8 % bits != 0)          */
+#define EXACT_E_SHAPE (-3)     /* negative / overflowing / unsupported size      */
+#define EXACT_E_ALIGN (-4)     /* pointer alignment the kernel needs is missing  */
+#define EXACT_E_ARG (-5)       /* any other bad argument (reduce, idx_bytes, p)  */
+
+#define EXACT_REDUCE_SUM 0
+#define EXACT_REDUCE_MEAN 1
+
+int exact_abi_version(void);
+/* Static string for a return code (EXACT_E_* name or hipGetErrorString). */
+const char *exact_strerror(int code);
+
+/* Bytes of the packed stream for an [N, G] activation at `bits`:
+ * (bits * N_round * G + 8) / 8 with N_round = N rounded up to 8/bits rows --
+ * the allocation of pack_single_precision_cuda, quantization_cuda_kernel.cu:107-113
+ * (the final byte is padding; this library writes it as 0). */
+int64_t exact_packed_nbytes(int64_t N, int64_t G, int bits);
+
+/* a1. Per-row minimum and maximum of x[N, G] (row-major fp32).
+ * Replaces the two torch reductions of QScheme.compute_quantization_bits
+ * (qsheme.py:41-48) / no_scheme_compute_quantization_bits (ops.py:61-66). */
+int exact_row_minmax_f32(const float *x, int64_t N, int64_t G,
+                         float *mn, float *mx, void *stream);
+
+/* a3. Stochastic-rounding quantise + bit-pack with caller-supplied per-row
+ * min and scale: replaces pack_single_precision(data, min, max, scale, bits,
+ * stochastic) (quantization.cc:37-48 -> quantization_cuda_kernel.cu:63-155).
+ *   q = rn(fmax((x - mn[n]) * scale[n] + u - 0.5, 0)), unfused fp32;
+ *   byte[(n / wpt) * G + d] |= q << ((n % wpt) * bits), wpt = 8 / bits.
+ * noise: fp32 [N, G] uniforms to use as u, or NULL to draw u from the
+ * library's Philox4x32-10 stream keyed by (seed, offset) (16 random bits per
+ * element, u = (h + 0.5) / 65536; counter = (d / 8, n, offset_lo, offset_hi)).
+ * packed must hold exact_packed_nbytes(N, G, bits) bytes. */
+int exact_pack_f32(const float *x, const float *mn, const float *scale,
+                   const float *noise, uint64_t seed, uint64_t offset,
+                   int64_t N, int64_t G, int bits, uint8_t *packed, void *stream);
+
+/* a1+a2+a3(+a4) fused: one read of x produces per-row min, scale =
+ * (2^bits - 1) / (max - min) (ops.py:39), the packed stream, and optionally
+ * the bf16 copies that quantize_activation returns (ops.py:80-81).
+ * Any of scale_f32 / min_f32 / scale_bf16 / min_bf16 may be NULL (skipped),
+ * except that rows longer than 1024 columns need scale_f32 and min_f32.
+ * Replaces quantize_activation's chain ops.py:69-83. */
+int exact_minmax_pack_f32(const float *x, const float *noise, uint64_t seed,
+                          uint64_t offset, int64_t N, int64_t G, int bits,
+                          uint8_t *packed, float *scale_f32, float *min_f32,
+                          uint16_t *scale_bf16, uint16_t *min_bf16, void *stream);
+
+/* a5. Unpack + dequantise: out[n, d] = float(field) / scale[n] + mn[n].
+ * Replaces unpack_single_precision(data, bits, scale, min, N, group_size)
+ * (quantization.cc:50-62 -> quantization_cuda_kernel.cu:158-229). */
+int exact_unpack_f32(const uint8_t *packed, int bits, const float *scale,
+                     const float *mn, int64_t N, int64_t G, float *out, void *stream);
+
+/* a6. Same with scale / min given as bf16 bit patterns (what
+ * quantize_activation returned): folds the bf16 -> fp32 widening of
+ * dequantize_activation (ops.py:92-98) into the kernel. */
+int exact_unpack_bf16param_f32(const uint8_t *packed, int bits,
+                               const uint16_t *scale_bf16, const uint16_t *min_bf16,
+                               int64_t N, int64_t G, float *out, void *stream);
+
+/* a13. ReLU that keeps a 1-bit mask: y = x > 0 ? x : 0; bit (i % 32) of
+ * mask[i / 32] = (x[i] > 0).  mask holds (n + 31) / 32 int32 words, all of
+ * them fully written.  Replaces act_quantized_relu_forward_cuda /
+ * act_quantized_relu_backward_cuda (quantization_cuda_kernel.cu:237-331). */
+int exact_relu_fwd_f32(const float *x, int64_t n, float *y, uint32_t *mask, void *stream);
+int exact_relu_bwd_f32(const float *dy, const uint32_t *mask, int64_t n, float *dx, void *stream);
+
+/* a14. Dropout that keeps a 1-bit keep mask: keep = u > p,
+ * y = x * keep * (1 / (1 - p)); backward dx = keep ? dy / (1 - p) : 0.
+ * noise NULL -> Philox (counter = (i / 8, offset)).  0 <= p < 1.
+ * Replaces act_quantized_dropout_forward_cuda / _backward_cuda
+ * (quantization_cuda_kernel.cu:442-594; quantization.cc:111-134). */
+int exact_dropout_fwd_f32(const float *x, const float *noise, uint64_t seed,
+                          uint64_t offset, float p, int64_t n, float *y,
+                          uint32_t *mask, void *stream);
+int exact_dropout_bwd_f32(const float *dy, const uint32_t *mask, float p,
+                          int64_t n, float *dx, void *stream);
+
+/* a10 / a11. CSR SpMM out[M, K] = reduce_{e in row r} val[e] * X[col[e], :].
+ * rowptr has M + 1 entries, col / val have nnz; idx_bytes is 4 (int32) or 8
+ * (int64) for both index arrays; val may be NULL (implicit ones); X is
+ * [n_cols, K] row-major fp32; nnz = rowptr[M] (passed in so the host never
+ * reads device memory); reduce is EXACT_REDUCE_SUM or _MEAN (mean divides by
+ * max(row length, 1)).  The entry stream is cut into equal chunks, one per
+ * wavefront, so hub rows are split across wavefronts.  Replaces spmm_cuda (spmm_cuda.cu:106-170,
+ * kernel :27-104, Reducer reducer.cuh:43-85); the backward products of
+ * spmm_sum_bw / spmm_mean_bw (spmm.cc:57-79, 115-139) are the same call on
+ * the CSC arrays. */
+int exact_spmm_csr_f32(const void *rowptr, const void *col, const float *val,
+                       int idx_bytes, const float *X, int64_t M, int64_t n_cols,
+                       int64_t K, int64_t nnz, int reduce, float *out, void *stream);
+
+/* a7. Random projection: out[N, k] = X[N, D] . R[D, k]  (input2rp, ops.py:107-118)
+ * and back: out[N, D] = Xr[N, k] . R[D, k]^T  (rp2input, ops.py:121-125).
+ * fp32 in, fp32 accumulate on the matrix cores. */
+int exact_rp_fwd_f32(const float *X, const float *R, int64_t N, int64_t D,
+                     int64_t k, float *out, void *stream);
+int exact_rp_bwd_f32(const float *Xr, const float *R, int64_t N, int64_t D,
+                     int64_t k, float *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EXACT_HIP_H_ */

@@ -1,0 +1,38 @@
+"""Helpers shared by the GPU parity tests."""
+import numpy as np
+import torch
+
+
+def dev(a, device="cuda:0"):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def host_noise(shape, seed):
+    """Uniform [0, 1) noise generated on the HOST with a seeded torch generator,
+    so the oracle and the kernels see identical bits."""
+    g = torch.Generator().manual_seed(seed)
+    return torch.rand(shape, generator=g, dtype=torch.float32).numpy()
+
+
+def host_randn(shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g, dtype=torch.float32).numpy()
+
+
+class FixedNoise:
+    """config.noise_source that hands out pre-made tensors in call order."""
+
+    def __init__(self, tensors):
+        self.tensors = list(tensors)
+        self.i = 0
+
+    def __call__(self, shape, device):
+        t = self.tensors[self.i]
+        self.i += 1
+        assert tuple(t.shape) == tuple(shape) or t.numel() == int(np.prod(shape))
+        return t.to(device).contiguous()
+
+
+def bytes_equal(t, arr):
+    a = t.detach().cpu().numpy()
+    return np.array_equal(a.view(np.uint8).reshape(-1), np.ascontiguousarray(arr).view(np.uint8).reshape(-1))
