@@ -197,4 +197,6 @@ class ActQuantizedDropout(torch.autograd.Function):
 def act_quantized_dropout(input, p, train):  # noqa: A002
     """quantization.cc:131-134."""
     check_device_tensor(input, "input")
+    if not train:
+        return input                      # quantization.cc:115-117
     return ActQuantizedDropout.apply(input, p, train)

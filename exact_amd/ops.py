@@ -94,7 +94,7 @@ def quantize_activation(input, scheme):  # noqa: A002
     check_device_tensor(input, "input")
     N = input.shape[0]
     q_bits = config.activation_compression_bits[0]
-    q_input, q_scale, q_min = ext_quantization.minmax_pack(input.view(N, -1), q_bits)
+    q_input, q_scale, q_min = ext_quantization.minmax_pack(input.reshape(N, input[0].numel() if N else int(np.prod(input.shape[1:]))), q_bits)
     if config.swap:
         q_input = swap_to_cpu(q_input)
     return q_input, q_bits, q_scale, q_min

@@ -24,6 +24,8 @@ def lib():
         _lib = ctypes.CDLL(LIB_PATH)
         _lib.oracle_packed_nbytes.restype = ctypes.c_int64
         _lib.oracle_packed_nbytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
+        _lib.oracle_count_fast_division_mismatches.restype = ctypes.c_int64
+        _lib.oracle_count_fast_division_mismatches.argtypes = [ctypes.c_int]
         _lib.oracle_f32_to_bf16.restype = ctypes.c_uint16
         _lib.oracle_f32_to_bf16.argtypes = [ctypes.c_float]
     return _lib

@@ -79,12 +79,14 @@ void oracle_row_minmax(const float *x, int64_t N, int64_t G, float *mn, float *m
   }
 }
 
-/* a2: scale = (2^b - 1) / (mx - mn), fp32 (ops.py:39) */
+/* a2: scale = (2^b - 1) / (mx - mn) (ops.py:39): int / tensor is
+ * tensor.reciprocal() * int in torch, i.e. two fp32 roundings */
 void oracle_scale(const float *mn, const float *mx, int64_t N, int bits, float *scale) {
   const float B = (float)((1 << bits) - 1);
   for (int64_t n = 0; n < N; ++n) {
     const float range = mx[n] - mn[n];
-    scale[n] = B / range;
+    const float recip = 1.0f / range;
+    scale[n] = recip * B;
   }
 }
 
@@ -281,4 +283,30 @@ void oracle_rp_bwd(const float *Xr, const float *R, int64_t N, int64_t D, int64_
       out[n * D + d] = acc;
     }
   }
+}
+
+/* ---- division identity used by the GPU unpack kernel ---------------------
+ * Counts the (significand of s, q) pairs, over ALL 2^23 significands at the
+ * given biased exponent and q = 0..255, for which
+ *   y = RN(q r), e = fma(-y, s, q), RN(y + e r)   with r = RN(1 / s)
+ * differs from the IEEE quotient q / s.  The kernel relies on the answer
+ * being 0; tests/test_oracle.py runs this. */
+int64_t oracle_count_fast_division_mismatches(int biased_exponent) {
+  int64_t bad = 0;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+  for (int64_t m = 0; m < (1 << 23); ++m) {
+    const uint32_t bits = ((uint32_t)biased_exponent << 23) | (uint32_t)m;
+    float s;
+    memcpy(&s, &bits, 4);
+    const float r = 1.0f / s;
+    for (int q = 0; q <= 255; ++q) {
+      const float qf = (float)q;
+      const float y = qf * r;
+      const float e = fmaf(-y, s, qf);
+      const float got = fmaf(e, r, y);
+      const float want = qf / s;
+      bad += memcmp(&got, &want, 4) != 0;
+    }
+  }
+  return bad;
 }

@@ -136,10 +136,14 @@ def row_min_max(x: np.ndarray):
     return x2.min(axis=1), x2.max(axis=1)
 
 
-# a2: scale = (2^b - 1) / (mx - mn) in fp32      (ops.py:39)
+# a2: scale = (2 ** bits - 1) / (mx - mn)      (ops.py:39)
 def compute_scale(mn: np.ndarray, mx: np.ndarray, bits: int) -> np.ndarray:
+    """`python_int / tensor` is Tensor.__rtruediv__, which torch defines as
+    `tensor.reciprocal() * python_int`: TWO fp32 roundings (1/range, then * B),
+    not one division.  Pinned by test_oracle.py against torch on the CPU."""
     with np.errstate(divide="ignore", invalid="ignore"):
-        return (F32(2 ** bits - 1) / (mx.astype(F32) - mn.astype(F32))).astype(F32)
+        recip = (F32(1.0) / (mx.astype(F32) - mn.astype(F32))).astype(F32)
+        return (recip * F32(2 ** bits - 1)).astype(F32)
 
 
 def packed_nbytes(N: int, G: int, bits: int) -> int:

@@ -34,5 +34,8 @@ class FixedNoise:
 
 
 def bytes_equal(t, arr):
-    a = t.detach().cpu().numpy()
+    t = t.detach().cpu()
+    if t.dtype == torch.bfloat16:
+        t = t.view(torch.int16)
+    a = t.numpy()
     return np.array_equal(a.view(np.uint8).reshape(-1), np.ascontiguousarray(arr).view(np.uint8).reshape(-1))

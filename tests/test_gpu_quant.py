@@ -144,7 +144,16 @@ def test_full_size_properties(cuda, bits):
     assert torch.equal(s32, (2 ** bits - 1) / (x.max(1).values - x.min(1).values))
     xh = extq.unpack_single_precision(packed, bits, s32, m32, N, G)
     step = 1.0 / s32.view(-1, 1)
-    assert ((xh - x).abs() <= step * 1.0001).all()
+    viol = (xh - x).abs() > step * 1.0001
+    # The reference has no upper clamp: when fp32 rounding makes (max - min) * scale
+    # exceed B and the noise is within an ulp of 1, the row maximum quantises to B + 1,
+    # which at 8 bits wraps to 0 in the byte.  Expected about once per 10^8 elements;
+    # anything else outside one quantisation step is a bug.
+    assert int(viol.sum()) <= 4
+    assert torch.equal(x[viol], x.max(1, keepdim=True).values.expand_as(x)[viol])
+    # every one of the 43 M dequantised values, bit for bit (the kernel divides once per row)
+    assert bytes_equal(xh, o.unpack_single_precision(packed.cpu().numpy(), bits, s32.cpu().numpy(),
+                                                     m32.cpu().numpy(), N, G))
     # re-quantising x_hat with noise == 0.5 (pure rounding) must reproduce the same codes
     config.noise_source = FixedNoise([torch.full_like(x, 0.5)])
     packed2 = extq.pack_single_precision(xh, m32, x.max(1).values, s32, bits, True)

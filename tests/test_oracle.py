@@ -201,6 +201,30 @@ def test_stochastic_rounding_is_unbiased():
     assert abs(u.mean() - 0.5) < 1e-3 and abs(u.var() - 1 / 12) < 1e-3
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_scale_is_reciprocal_times_B_like_torch(bits):
+    """ops.py:39 is `(2 ** bits - 1) / (mx - mn)` on tensors: torch evaluates
+    int / tensor as tensor.reciprocal() * int (two roundings)."""
+    rng = np.random.default_rng(bits)
+    mn = rng.standard_normal(20000).astype(F32)
+    mx = (mn + np.abs(rng.standard_normal(20000)).astype(F32) * F32(3)).astype(F32)
+    mx[0] = mn[0]
+    want = ((2 ** bits - 1) / (torch.from_numpy(mx) - torch.from_numpy(mn))).numpy()
+    assert np.array_equal(o.compute_scale(mn, mx, bits).view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(co.scale(mn, mx, bits).view(np.uint32), want.view(np.uint32))
+    if bits > 1:   # and it is NOT the single division
+        single = (F32(2 ** bits - 1) / (mx[1:] - mn[1:])).astype(F32)
+        assert not np.array_equal(single, want[1:])
+
+
+def test_fast_division_identity_exhaustive():
+    """The unpack kernel divides once per row and corrects per element; the
+    correction is exact for every significand (one exponent is exhaustive for
+    the normal range, two more guard against an exponent dependence)."""
+    for e in (127, 64, 190):
+        assert co.lib().oracle_count_fast_division_mismatches(e) == 0
+
+
 # ------------------------------------------------------------------ masks ---
 def test_relu_matches_torch_autograd():
     rng = np.random.default_rng(1)
