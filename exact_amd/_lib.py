@@ -10,7 +10,8 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libexact_hip.so")
+# EXACT_AMD_LIB overrides the path (e.g. to load a differently built library)
+LIB_PATH = os.environ.get("EXACT_AMD_LIB") or os.path.join(_HERE, "libexact_hip.so")
 
 _c_i64 = ctypes.c_int64
 _c_u64 = ctypes.c_uint64
@@ -55,6 +56,13 @@ def lib() -> ctypes.CDLL:
                     raise ExactLibraryError(
                         f"{LIB_PATH} is missing: build it with `python -m exact_amd.build` "
                         "(hipcc, gfx950). exact_amd has no fallback path.")
+                # torch must bring up its HIP runtime first: the library then binds
+                # to that same runtime (one libamdhip64 per process), and a library
+                # loaded ahead of torch's device initialisation has left torch
+                # unable to see the GPU.
+                import torch
+                if torch.cuda.is_available():
+                    torch.cuda.init()
                 handle = ctypes.CDLL(LIB_PATH)
                 for name, (res, args) in SIGNATURES.items():
                     fn = getattr(handle, name)  # AttributeError if the symbol is not exported

@@ -9,10 +9,15 @@ def _fail(msg):
     raise RuntimeError(msg)
 
 
+def on_device(t):
+    """True for tensors the kernels may touch (device memory)."""
+    return t.is_cuda
+
+
 def check_device_tensor(t, name, dim=None, dtypes=(torch.float32,)):
     if not isinstance(t, torch.Tensor):
         _fail(f"{name} must be a tensor!")
-    if not t.is_cuda:
+    if not on_device(t):
         _fail(f"{name} must be a CUDA tensor!")
     if not t.is_contiguous():
         _fail(f"{name} must be contiguous!")

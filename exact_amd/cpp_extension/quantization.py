@@ -13,7 +13,8 @@ import torch
 from .. import _lib
 from ..conf import config
 from ..rng import next_philox
-from ._checks import check_device_tensor, ptr, stream_ptr
+from . import _checks
+from ._checks import check_device_tensor, ptr
 
 
 def packed_nbytes(N: int, G: int, bits: int) -> int:
@@ -55,7 +56,7 @@ def pack_single_precision(data, min, max, scale, bits, stochastic):  # noqa: A00
     packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=data.device)
     noise, seed, offset = _noise_for(data.shape, data.device)
     rc = _lib.lib().exact_pack_f32(ptr(data), ptr(min), ptr(scale), ptr(noise), seed, offset,
-                                   N, G, bits, ptr(packed), stream_ptr(data))
+                                   N, G, bits, ptr(packed), _checks.stream_ptr(data))
     _lib.check(rc, "pack_single_precision")
     return packed
 
@@ -70,7 +71,7 @@ def unpack_single_precision(data, bits, scale, min, N, group_size):  # noqa: A00
     if data.numel() < packed_nbytes(N, G, bits) - 1 or scale.numel() < N or min.numel() < N:
         raise RuntimeError("packed data / scale / min are too short for N x group_size")
     out = torch.empty((N, G), dtype=scale.dtype, device=data.device)
-    rc = _lib.lib().exact_unpack_f32(ptr(data), bits, ptr(scale), ptr(min), N, G, ptr(out), stream_ptr(data))
+    rc = _lib.lib().exact_unpack_f32(ptr(data), bits, ptr(scale), ptr(min), N, G, ptr(out), _checks.stream_ptr(data))
     _lib.check(rc, "unpack_single_precision")
     return out
 
@@ -93,7 +94,7 @@ def minmax_pack(data, bits, want_fp32=False):
     noise, seed, offset = _noise_for(data.shape, dev)
     rc = _lib.lib().exact_minmax_pack_f32(ptr(data), ptr(noise), seed, offset, N, G, bits, ptr(packed),
                                           ptr(scale32), ptr(min32), ptr(scale_bf), ptr(min_bf),
-                                          stream_ptr(data))
+                                          _checks.stream_ptr(data))
     _lib.check(rc, "minmax_pack")
     if want_fp32:
         return packed, scale_bf, min_bf, scale32, min32
@@ -112,7 +113,7 @@ def unpack_bf16param(data, bits, scale_bf16, min_bf16, N, group_size):
         raise RuntimeError("packed data / scale / min are too short for N x group_size")
     out = torch.empty((N, G), dtype=torch.float32, device=data.device)
     rc = _lib.lib().exact_unpack_bf16param_f32(ptr(data), bits, ptr(scale_bf16), ptr(min_bf16), N, G,
-                                               ptr(out), stream_ptr(data))
+                                               ptr(out), _checks.stream_ptr(data))
     _lib.check(rc, "unpack_bf16param")
     return out
 
@@ -122,7 +123,7 @@ def row_minmax(data):
     N, G = data.shape
     mn = torch.empty(N, dtype=torch.float32, device=data.device)
     mx = torch.empty(N, dtype=torch.float32, device=data.device)
-    rc = _lib.lib().exact_row_minmax_f32(ptr(data), N, G, ptr(mn), ptr(mx), stream_ptr(data))
+    rc = _lib.lib().exact_row_minmax_f32(ptr(data), N, G, ptr(mn), ptr(mx), _checks.stream_ptr(data))
     _lib.check(rc, "row_minmax")
     return mn, mx
 
@@ -140,7 +141,7 @@ class ActQuantizedReLU(torch.autograd.Function):
         n = input.numel()
         out = torch.empty_like(input)
         mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
-        rc = _lib.lib().exact_relu_fwd_f32(ptr(input), n, ptr(out), ptr(mask), stream_ptr(input))
+        rc = _lib.lib().exact_relu_fwd_f32(ptr(input), n, ptr(out), ptr(mask), _checks.stream_ptr(input))
         _lib.check(rc, "act_quantized_relu")
         ctx.save_for_backward(mask)
         return out
@@ -151,7 +152,7 @@ class ActQuantizedReLU(torch.autograd.Function):
         grad_output = grad_output.contiguous()
         grad_input = torch.empty_like(grad_output)
         rc = _lib.lib().exact_relu_bwd_f32(ptr(grad_output), ptr(mask), grad_output.numel(),
-                                           ptr(grad_input), stream_ptr(grad_output))
+                                           ptr(grad_input), _checks.stream_ptr(grad_output))
         _lib.check(rc, "act_quantized_relu backward")
         return grad_input
 
@@ -174,7 +175,7 @@ class ActQuantizedDropout(torch.autograd.Function):
         mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
         noise, seed, offset = _noise_for(input.shape, input.device)
         rc = _lib.lib().exact_dropout_fwd_f32(ptr(input), ptr(noise), seed, offset, float(p), n,
-                                              ptr(out), ptr(mask), stream_ptr(input))
+                                              ptr(out), ptr(mask), _checks.stream_ptr(input))
         _lib.check(rc, "act_quantized_dropout")
         ctx.save_for_backward(mask)
         ctx.p = float(p)
@@ -189,7 +190,7 @@ class ActQuantizedDropout(torch.autograd.Function):
         grad_output = grad_output.contiguous()
         grad_input = torch.empty_like(grad_output)
         rc = _lib.lib().exact_dropout_bwd_f32(ptr(grad_output), ptr(mask), ctx.p, grad_output.numel(),
-                                              ptr(grad_input), stream_ptr(grad_output))
+                                              ptr(grad_input), _checks.stream_ptr(grad_output))
         _lib.check(rc, "act_quantized_dropout backward")
         return grad_input, None, None
 

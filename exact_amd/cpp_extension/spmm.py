@@ -10,13 +10,14 @@ from collections import OrderedDict
 import torch
 
 from .. import _lib
-from ._checks import ptr, stream_ptr
+from . import _checks
+from ._checks import ptr
 
 REDUCE = {"sum": 0, "mean": 1}
 
 
 def _check_index(t, name):
-    if not t.is_cuda:
+    if not _checks.on_device(t):
         raise RuntimeError(f"{name} must be CUDA tensor")       # CHECK_CUDA, spmm_cuda.cu:111-116
     if t.dim() != 1:
         raise RuntimeError("Input mismatch")                     # CHECK_INPUT, spmm_cuda.cu:118-119
@@ -31,14 +32,14 @@ def spmm_csr(rowptr, col, value, mat, reduce):
         raise NotImplementedError(f"reduce='{reduce}' is not implemented by this library (sum, mean only)")
     _check_index(rowptr, "rowptr")
     _check_index(col, "col")
-    if not mat.is_cuda:
+    if not _checks.on_device(mat):
         raise RuntimeError("mat must be CUDA tensor")
     if mat.dim() != 2:
         raise RuntimeError("Input mismatch: mat must be 2-D [N, K]")
     if mat.dtype != torch.float32:
         raise RuntimeError("The type of mat is not correct!")
     if value is not None:
-        if not value.is_cuda:
+        if not _checks.on_device(value):
             raise RuntimeError("value must be CUDA tensor")
         if value.dim() != 1 or value.size(0) != col.size(0):
             raise RuntimeError("Input mismatch")                 # spmm_cuda.cu:121-122
@@ -53,7 +54,7 @@ def spmm_csr(rowptr, col, value, mat, reduce):
     n_cols, K = mat.shape
     out = torch.empty((M, K), dtype=mat.dtype, device=mat.device)
     rc = _lib.lib().exact_spmm_csr_f32(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat),
-                                       M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out), stream_ptr(mat))
+                                       M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out), _checks.stream_ptr(mat))
     _lib.check(rc, f"spmm_{reduce}")
     return out
 

@@ -8,88 +8,109 @@
 // element i, every word of the (n + 31) / 32-word mask is written in full, and
 // nothing is written past it.
 //
-// Each lane owns one oct (8 consecutive elements, 32 B): its 8 mask bits are
-// one byte, and four neighbouring lanes merge their bytes into the 32-bit
-// mask word with two cross-lane ORs.
+// Each lane owns two quads (4 consecutive elements, one 16-byte access each):
+// quad t and quad t + 256 of its workgroup's 512-quad tile, so every vector
+// memory instruction of a wavefront covers 1 KiB of consecutive addresses.
+// The 4 mask bits of a quad are a nibble; eight neighbouring lanes merge their
+// nibbles into one 32-bit mask word with three DPP ORs.  Dropout noise comes
+// from one Philox block per 8 consecutive elements: the even lane of a lane
+// pair draws the block of the pair's first quad, the odd lane that of its
+// second quad, and the two trade halves.
 
 #include "exact_common.hpp"
 
 namespace exact {
 
+constexpr int kTileQuads = 2 * kBlock;  // quads per workgroup
+
 template <bool VEC4>
-__device__ __forceinline__ void load8(const float* __restrict__ p, int nv, float (&v)[8]) {
-  if (VEC4 && nv == 8) {
+__device__ __forceinline__ void load4(const float* __restrict__ p, int nv, float (&v)[4]) {
+  if (VEC4 && nv == 4) {
     const f32x4 a = nt_load4(p);
-    const f32x4 b = nt_load4(p + 4);
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (i < nv) ? p[i] : 0.f;
+    for (int i = 0; i < 4; ++i) v[i] = (i < nv) ? p[i] : 0.f;
   }
 }
 
 template <bool VEC4>
-__device__ __forceinline__ void store8(float* __restrict__ p, int nv, const float (&v)[8]) {
-  if (VEC4 && nv == 8) {
+__device__ __forceinline__ void store4(float* __restrict__ p, int nv, const float (&v)[4]) {
+  if (VEC4 && nv == 4) {
     nt_store4(p, v[0], v[1], v[2], v[3]);
-    nt_store4(p + 4, v[4], v[5], v[6], v[7]);
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 4; ++i)
       if (i < nv) p[i] = v[i];
   }
 }
 
-// Merge the mask bytes of lanes 4m..4m+3 into one word; lane 4m stores it.
-__device__ __forceinline__ void store_mask_byte(uint32_t byte, int64_t oct, int64_t n,
-                                                uint32_t* __restrict__ mask) {
-  uint32_t w = byte << (8 * (threadIdx.x & 3));
-  w |= __shfl_xor(w, 1);
-  w |= __shfl_xor(w, 2);
-  if ((threadIdx.x & 3) == 0 && oct * 8 < n) mask[oct >> 2] = w;
+__device__ __forceinline__ int valid_in_quad(int64_t quad, int64_t n) {
+  const int64_t left = n - quad * 4;
+  return left >= 4 ? 4 : (left > 0 ? static_cast<int>(left) : 0);
 }
 
-__device__ __forceinline__ uint32_t load_mask_byte(const uint32_t* __restrict__ mask, int64_t oct) {
-  return (mask[oct >> 2] >> (8 * (oct & 3))) & 0xFFu;
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), CTRL, 0xF, 0xF, true));
+}
+
+// OR the nibbles of lanes 8m..8m+7 into one mask word; lane 8m stores it.
+// quad_perm [1,0,3,2] and [2,3,0,1] fold within groups of four lanes, the
+// half-row mirror (lane i <-> 7 - i) then folds the two groups.
+__device__ __forceinline__ void store_mask_nibble(uint32_t nibble, int64_t quad, int64_t n,
+                                                  uint32_t* __restrict__ mask) {
+  uint32_t w = nibble << (4 * (threadIdx.x & 7));
+  w |= dpp<0xB1>(w);
+  w |= dpp<0x4E>(w);
+  w |= dpp<0x141>(w);
+  if ((threadIdx.x & 7) == 0 && quad * 4 < n) mask[quad >> 3] = w;
+}
+
+__device__ __forceinline__ uint32_t load_mask_nibble(const uint32_t* __restrict__ mask, int64_t quad) {
+  return (mask[quad >> 3] >> (4 * (quad & 7))) & 0xFu;
 }
 
 template <bool VEC4>
 __global__ __launch_bounds__(kBlock) void relu_fwd_kernel(const float* __restrict__ x, int64_t n,
                                                           float* __restrict__ y,
                                                           uint32_t* __restrict__ mask) {
-  const int64_t oct = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const int64_t left = n - oct * 8;
-  const int nv = left >= 8 ? 8 : (left > 0 ? static_cast<int>(left) : 0);
-  float v[8];
-  uint32_t byte = 0;
-  if (nv > 0) {
-    load8<VEC4>(x + oct * 8, nv, v);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const bool bit = v[i] > 0.f;  // quantization_cuda_kernel.cu:252-257
-      v[i] = bit ? v[i] : 0.f;
-      byte |= static_cast<uint32_t>(bit && i < nv) << i;
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
+    const int nv = valid_in_quad(quad, n);
+    float v[4];
+    uint32_t nibble = 0;
+    if (nv > 0) {
+      load4<VEC4>(x + quad * 4, nv, v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool bit = v[i] > 0.f;  // quantization_cuda_kernel.cu:252-257
+        v[i] = bit ? v[i] : 0.f;
+        nibble |= static_cast<uint32_t>(bit && i < nv) << i;
+      }
+      store4<VEC4>(y + quad * 4, nv, v);
     }
-    store8<VEC4>(y + oct * 8, nv, v);
+    store_mask_nibble(nibble, quad, n, mask);
   }
-  store_mask_byte(byte, oct, n, mask);
 }
 
 template <bool VEC4>
 __global__ __launch_bounds__(kBlock) void relu_bwd_kernel(const float* __restrict__ dy,
                                                           const uint32_t* __restrict__ mask, int64_t n,
                                                           float* __restrict__ dx) {
-  const int64_t oct = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const int64_t left = n - oct * 8;
-  if (left <= 0) return;
-  const int nv = left >= 8 ? 8 : static_cast<int>(left);
-  float v[8];
-  load8<VEC4>(dy + oct * 8, nv, v);
-  const uint32_t byte = load_mask_byte(mask, oct);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = ((byte >> i) & 1u) ? v[i] : 0.f;  // :305-310
-  store8<VEC4>(dx + oct * 8, nv, v);
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
+    const int nv = valid_in_quad(quad, n);
+    if (nv == 0) continue;
+    float v[4];
+    load4<VEC4>(dy + quad * 4, nv, v);
+    const uint32_t nibble = load_mask_nibble(mask, quad);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = ((nibble >> i) & 1u) ? v[i] : 0.f;  // :305-310
+    store4<VEC4>(dx + quad * 4, nv, v);
+  }
 }
 
 template <bool VEC4, bool NOISE_IN>
@@ -99,56 +120,71 @@ __global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const float* __rest
                                                              uint32_t off_lo, uint32_t off_hi, float p,
                                                              float pinv, int64_t n, float* __restrict__ y,
                                                              uint32_t* __restrict__ mask) {
-  const int64_t oct = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const int64_t left = n - oct * 8;
-  const int nv = left >= 8 ? 8 : (left > 0 ? static_cast<int>(left) : 0);
-  uint32_t byte = 0;
-  if (nv > 0) {
-    float v[8], u[8];
-    load8<VEC4>(x + oct * 8, nv, v);
-    if constexpr (NOISE_IN) {
-      load8<VEC4>(noise + oct * 8, nv, u);
-    } else {
-      const Philox4 r = philox4x32_10(static_cast<uint32_t>(oct), static_cast<uint32_t>(oct >> 32),
-                                      off_lo, off_hi, seed_lo, seed_hi);
-      philox_uniform8(r, u);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const bool keep = u[i] > p;  // quantization_cuda_kernel.cu:465-468
-      const float kf = keep ? 1.f : 0.f;
-      float r = v[i] * kf;  // :490, left to right
-      r = r * pinv;
-      v[i] = r;
-      byte |= static_cast<uint32_t>(keep && i < nv) << i;
-    }
-    store8<VEC4>(y + oct * 8, nv, v);
+  const int64_t qa = static_cast<int64_t>(blockIdx.x) * kTileQuads + threadIdx.x;
+  const int64_t qb = qa + kBlock;
+  float u[2][4];
+  if constexpr (!NOISE_IN) {
+    // flat element i draws from block i / 8 = quad / 2: counter (block lo, block hi, offset)
+    const bool odd = (threadIdx.x & 1) != 0;
+    const int64_t blk = (odd ? qb : qa) >> 1;
+    const Philox4 r = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32), off_lo, off_hi,
+                                    seed_lo, seed_hi);
+    const uint32_t got0 = dpp<0xB1>(odd ? r.x : r.z);
+    const uint32_t got1 = dpp<0xB1>(odd ? r.y : r.w);
+    const uint32_t a0 = odd ? got0 : r.x, a1 = odd ? got1 : r.y;
+    const uint32_t b0 = odd ? r.z : got0, b1 = odd ? r.w : got1;
+    u[0][0] = u16_to_uniform(a0 & 0xFFFFu); u[0][1] = u16_to_uniform(a0 >> 16);
+    u[0][2] = u16_to_uniform(a1 & 0xFFFFu); u[0][3] = u16_to_uniform(a1 >> 16);
+    u[1][0] = u16_to_uniform(b0 & 0xFFFFu); u[1][1] = u16_to_uniform(b0 >> 16);
+    u[1][2] = u16_to_uniform(b1 & 0xFFFFu); u[1][3] = u16_to_uniform(b1 >> 16);
   }
-  store_mask_byte(byte, oct, n, mask);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = h ? qb : qa;
+    const int nv = valid_in_quad(quad, n);
+    uint32_t nibble = 0;
+    if (nv > 0) {
+      float v[4];
+      load4<VEC4>(x + quad * 4, nv, v);
+      if constexpr (NOISE_IN) load4<VEC4>(noise + quad * 4, nv, u[h]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool keep = u[h][i] > p;  // quantization_cuda_kernel.cu:465-468
+        const float kf = keep ? 1.f : 0.f;
+        float r = v[i] * kf;  // :490, left to right
+        r = r * pinv;
+        v[i] = r;
+        nibble |= static_cast<uint32_t>(keep && i < nv) << i;
+      }
+      store4<VEC4>(y + quad * 4, nv, v);
+    }
+    store_mask_nibble(nibble, quad, n, mask);
+  }
 }
 
 template <bool VEC4>
 __global__ __launch_bounds__(kBlock) void dropout_bwd_kernel(const float* __restrict__ dy,
                                                              const uint32_t* __restrict__ mask, float p1m,
                                                              int64_t n, float* __restrict__ dx) {
-  const int64_t oct = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const int64_t left = n - oct * 8;
-  if (left <= 0) return;
-  const int nv = left >= 8 ? 8 : static_cast<int>(left);
-  float v[8];
-  load8<VEC4>(dy + oct * 8, nv, v);
-  const uint32_t byte = load_mask_byte(mask, oct);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = ((byte >> i) & 1u) ? v[i] / p1m : 0.f;  // :565-569
-  store8<VEC4>(dx + oct * 8, nv, v);
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
+    const int nv = valid_in_quad(quad, n);
+    if (nv == 0) continue;
+    float v[4];
+    load4<VEC4>(dy + quad * 4, nv, v);
+    const uint32_t nibble = load_mask_nibble(mask, quad);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = ((nibble >> i) & 1u) ? v[i] / p1m : 0.f;  // :565-569
+    store4<VEC4>(dx + quad * 4, nv, v);
+  }
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Octs rounded up to whole mask words (4 octs), then to workgroups.
-static dim3 oct_grid(int64_t n) {
-  const int64_t octs = ((n + 31) / 32) * 4;
-  return dim3(static_cast<unsigned>((octs + kBlock - 1) / kBlock));
+static dim3 tile_grid(int64_t n) {
+  const int64_t quads = (n + 3) / 4;
+  return dim3(static_cast<unsigned>((quads + kTileQuads - 1) / kTileQuads));
 }
 
 }  // namespace exact
@@ -163,9 +199,9 @@ int exact_relu_fwd_f32(const float* x, int64_t n, float* y, uint32_t* mask, void
   if (!x || !y || !mask) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (aligned16(x) && aligned16(y))
-    hipLaunchKernelGGL((relu_fwd_kernel<true>), oct_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
+    hipLaunchKernelGGL((relu_fwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
   else
-    hipLaunchKernelGGL((relu_fwd_kernel<false>), oct_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
+    hipLaunchKernelGGL((relu_fwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
   return launch_status();
 }
 
@@ -175,9 +211,9 @@ int exact_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float* 
   if (!dy || !dx || !mask) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (aligned16(dy) && aligned16(dx))
-    hipLaunchKernelGGL((relu_bwd_kernel<true>), oct_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
+    hipLaunchKernelGGL((relu_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
   else
-    hipLaunchKernelGGL((relu_bwd_kernel<false>), oct_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
+    hipLaunchKernelGGL((relu_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
   return launch_status();
 }
 
@@ -193,7 +229,7 @@ int exact_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uin
   const uint32_t sl = static_cast<uint32_t>(seed), sh = static_cast<uint32_t>(seed >> 32);
   const uint32_t ol = static_cast<uint32_t>(offset), oh = static_cast<uint32_t>(offset >> 32);
   const bool v4 = aligned16(x) && aligned16(y) && (!noise || aligned16(noise));
-  const dim3 grid = oct_grid(n);
+  const dim3 grid = tile_grid(n);
   if (noise) {
     if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, true>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
     else hipLaunchKernelGGL((dropout_fwd_kernel<false, true>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
@@ -214,9 +250,9 @@ int exact_dropout_bwd_f32(const float* dy, const uint32_t* mask, float p, int64_
   // quantization.cc:121,127: p1m = 1. - p stored as double, read back into a float
   const float p1m = static_cast<float>(1.0 - static_cast<double>(p));
   if (aligned16(dy) && aligned16(dx))
-    hipLaunchKernelGGL((dropout_bwd_kernel<true>), oct_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
+    hipLaunchKernelGGL((dropout_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
   else
-    hipLaunchKernelGGL((dropout_bwd_kernel<false>), oct_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
+    hipLaunchKernelGGL((dropout_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
   return launch_status();
 }
 

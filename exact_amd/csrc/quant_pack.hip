@@ -1,9 +1,8 @@
-// Per-row min/range, stochastic-rounding quantise + bit-pack, and the matching
-// unpack + dequantise, for [N, G] fp32 activations on gfx950.
+// Per-row min/range and stochastic-rounding quantise + bit-pack for [N, G]
+// fp32 activations on gfx950 (the matching unpack lives in quant_unpack.hip).
 //
 // Algorithm restated from the reference kernels
 //   pack_single_precision_kernel    quantization_cuda_kernel.cu:63-94
-//   unpack_single_precision_kernel  quantization_cuda_kernel.cu:158-185
 // and the torch glue around them (ops.py:20-98, qsheme.py:41-48); the
 // decomposition below is this library's own.
 //
@@ -249,102 +248,6 @@ __global__ __launch_bounds__(kBlock) void row_minmax_kernel(const float* __restr
 }
 
 // ---------------------------------------------------------------------------
-// unpack
-// ---------------------------------------------------------------------------
-struct UnpackArgs {
-  const uint8_t* packed;
-  const void* scale;  // float* or bf16 bits
-  const void* mn;
-  int64_t N;
-  int G;
-  int opr;
-  int lpr_log2;
-  int in_vec;  // 8, 4 or 1: widest aligned load of packed bytes
-  float* out;
-};
-
-// RN(q / s) from r = RN(1 / s): y = RN(q r), e = q - y s (exact, one FMA),
-// result = RN(y + e r).  Markstein's correction step; for 0 <= q <= 255 and
-// every fp32 significand of s it equals the IEEE quotient bit for bit (checked
-// exhaustively on the CPU: 2^23 significands x 256 values of q).
-__device__ __forceinline__ float exact_quotient(float q, float s, float r) {
-  const float y = q * r;
-  const float e = __fmaf_rn(-y, s, q);
-  return __fmaf_rn(e, r, y);
-}
-
-template <int BITS, int OPT, int VEC, bool FULL, bool BF16P>
-__global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
-  constexpr int WPT = 8 / BITS;
-  constexpr uint32_t FIELD = ((1u << BITS) - 1u) * 0x01010101u;
-  const int t = threadIdx.x;
-  const int lpr = 1 << a.lpr_log2;
-  const int lane_in_row = t & (lpr - 1);
-  const int rows_per_wg = kBlock >> a.lpr_log2;
-  const int64_t n = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (t >> a.lpr_log2);
-  if (n >= a.N) return;
-  const int oct_base = blockIdx.y * (lpr * OPT);
-
-  float sc, mnv;
-  if constexpr (BF16P) {
-    sc = bf16_to_f32(static_cast<const uint16_t*>(a.scale)[n]);
-    mnv = bf16_to_f32(static_cast<const uint16_t*>(a.mn)[n]);
-  } else {
-    sc = static_cast<const float*>(a.scale)[n];
-    mnv = static_cast<const float*>(a.mn)[n];
-  }
-  // One IEEE division per row instead of one per element: with rcp = RN(1/sc),
-  // exact_quotient() returns RN(q / sc) for every integer 0 <= q <= 255 as long
-  // as sc is a normal number far from the exponent limits; other rows divide.
-  const float asc = fabsf(sc);
-  const bool fast_div = asc >= 0x1p-64f && asc <= 0x1p64f;
-  const float rcp = 1.0f / sc;
-  const int shift = static_cast<int>(n & (WPT - 1)) * BITS;
-  const uint8_t* grp = a.packed + (n / WPT) * a.G;
-  float* orow = a.out + n * a.G;
-
-#pragma unroll
-  for (int k = 0; k < OPT; ++k) {
-    const int j = oct_base + lane_in_row + k * lpr;
-    if (!FULL && j >= a.opr) continue;
-    const int d0 = 8 * j;
-    const int nv = FULL ? 8 : min(8, a.G - d0);
-    uint32_t w0 = 0, w1 = 0;
-    if (FULL || a.in_vec == 8) {
-      const uint2 w = *reinterpret_cast<const uint2*>(grp + d0);
-      w0 = w.x;
-      w1 = w.y;
-    } else if (a.in_vec == 4) {
-      w0 = *reinterpret_cast<const uint32_t*>(grp + d0);
-      if (nv > 4) w1 = *reinterpret_cast<const uint32_t*>(grp + d0 + 4);
-    } else {
-      for (int i = 0; i < nv; ++i) {
-        const uint32_t byte = grp[d0 + i];
-        if (i < 4) w0 |= byte << (8 * i); else w1 |= byte << (8 * (i - 4));
-      }
-    }
-    w0 = (w0 >> shift) & FIELD;
-    w1 = (w1 >> shift) & FIELD;
-    float r[8];
-    if (__builtin_expect(fast_div, 1)) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float qf = static_cast<float>((i < 4 ? w0 >> (8 * i) : w1 >> (8 * (i - 4))) & 0xFFu);
-        r[i] = exact_quotient(qf, sc, rcp) + mnv;
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float qf = static_cast<float>((i < 4 ? w0 >> (8 * i) : w1 >> (8 * (i - 4))) & 0xFFu);
-        // quantization_cuda_kernel.cu:182: true division, then add
-        r[i] = qf / sc + mnv;
-      }
-    }
-    store_oct<VEC, FULL>(orow + d0, nv, r);
-  }
-}
-
-// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 struct Geometry {
@@ -479,46 +382,6 @@ static int pack_common(const float* x, const float* mn, const float* scale, cons
   return launch_status();
 }
 
-template <int BITS, bool BF16P>
-static void launch_unpack_variant(const UnpackArgs& a, bool vec4, bool full, dim3 grid, hipStream_t s) {
-  if (vec4 && full)
-    hipLaunchKernelGGL((unpack_kernel<BITS, 1, 4, true, BF16P>), grid, dim3(kBlock), 0, s, a);
-  else if (vec4)
-    hipLaunchKernelGGL((unpack_kernel<BITS, 1, 4, false, BF16P>), grid, dim3(kBlock), 0, s, a);
-  else
-    hipLaunchKernelGGL((unpack_kernel<BITS, 1, 1, false, BF16P>), grid, dim3(kBlock), 0, s, a);
-}
-
-template <bool BF16P>
-static int unpack_common(const uint8_t* packed, int bits, const void* scale, const void* mn,
-                         int64_t N, int64_t G, float* out, hipStream_t s) {
-  if (int rc = check_quant_shape(N, G, bits)) return rc;
-  if (N == 0 || G == 0) return EXACT_OK;
-  if (!packed || !scale || !mn || !out) return EXACT_E_NULL;
-  const Geometry g = plan_rows(G, 1);
-  UnpackArgs a;
-  a.packed = packed;
-  a.scale = scale;
-  a.mn = mn;
-  a.N = N;
-  a.G = static_cast<int>(G);
-  a.opr = g.opr;
-  a.lpr_log2 = g.lpr_log2;
-  a.out = out;
-  a.in_vec = (G % 8 == 0 && aligned(packed, 8)) ? 8 : (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
-  const bool vec4 = (G % 4 == 0) && aligned(out, 16);
-  const bool full = g.full && vec4 && a.in_vec == 8;
-  const int rows_per_wg = kBlock >> g.lpr_log2;
-  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(g.grid_y));
-  switch (bits) {
-    case 1: launch_unpack_variant<1, BF16P>(a, vec4, full, grid, s); break;
-    case 2: launch_unpack_variant<2, BF16P>(a, vec4, full, grid, s); break;
-    case 4: launch_unpack_variant<4, BF16P>(a, vec4, full, grid, s); break;
-    default: launch_unpack_variant<8, BF16P>(a, vec4, full, grid, s); break;
-  }
-  return launch_status();
-}
-
 }  // namespace exact
 
 using namespace exact;
@@ -561,16 +424,6 @@ int exact_minmax_pack_f32(const float* x, const float* noise, uint64_t seed, uin
                           float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, void* stream) {
   return pack_common(x, nullptr, nullptr, noise, seed, offset, N, G, bits, packed, scale_f32, min_f32,
                      scale_bf16, min_bf16, true, static_cast<hipStream_t>(stream));
-}
-
-int exact_unpack_f32(const uint8_t* packed, int bits, const float* scale, const float* mn, int64_t N,
-                     int64_t G, float* out, void* stream) {
-  return unpack_common<false>(packed, bits, scale, mn, N, G, out, static_cast<hipStream_t>(stream));
-}
-
-int exact_unpack_bf16param_f32(const uint8_t* packed, int bits, const uint16_t* scale_bf16,
-                               const uint16_t* min_bf16, int64_t N, int64_t G, float* out, void* stream) {
-  return unpack_common<true>(packed, bits, scale_bf16, min_bf16, N, G, out, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,197 @@
+// Unpack + dequantise of the packed activation stream for [N, G] fp32
+// activations on gfx950.
+//
+// Algorithm restated from the reference kernel
+//   unpack_single_precision_kernel  quantization_cuda_kernel.cu:158-185
+// and dequantize_activation (ops.py:86-98); the decomposition is this
+// library's own.
+//
+// Work unit: a "quad" = 4 consecutive columns of one row: one 32-bit load of
+// packed bytes (4 columns x 8/bits rows), one 16-byte store of fp32.  A row is
+// owned by `lpr` adjacent lanes (a power of two in [2, 32]); lane i of the row
+// handles quads i and i + lpr, so every vector store of a wavefront covers
+// whole contiguous runs of 16 * lpr bytes -- the kernel is bound by writing
+// the [N, G] fp32 output once.
+
+#include "exact_common.hpp"
+
+namespace exact {
+
+template <int VEC>
+__device__ __forceinline__ void store_quad(float* __restrict__ p, int nv, const float (&v)[4]) {
+  if constexpr (VEC == 4) {
+    if (nv > 0) nt_store4(p, v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < nv) __builtin_nontemporal_store(v[i], p + i);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// unpack
+// ---------------------------------------------------------------------------
+struct UnpackArgs {
+  const uint8_t* packed;
+  const void* scale;  // float* or bf16 bits
+  const void* mn;
+  int64_t N;
+  int G;
+  int qpr;
+  int lpr_log2;
+  int in_vec;  // 4 or 1: widest aligned load of packed bytes
+  float* out;
+};
+
+// RN(q / s) from r = RN(1 / s): y = RN(q r), e = q - y s (exact, one FMA),
+// result = RN(y + e r).  Markstein's correction step; for 0 <= q <= 255 and
+// every fp32 significand of s it equals the IEEE quotient bit for bit (checked
+// exhaustively on the CPU: 2^23 significands x 256 values of q).
+__device__ __forceinline__ float exact_quotient(float q, float s, float r) {
+  const float y = q * r;
+  const float e = __fmaf_rn(-y, s, q);
+  return __fmaf_rn(e, r, y);
+}
+
+template <int BITS, int SLOTS, int VEC, bool BF16P>
+__global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
+  constexpr int WPT = 8 / BITS;
+  constexpr uint32_t FIELD = ((1u << BITS) - 1u) * 0x01010101u;
+  const int t = threadIdx.x;
+  const int lpr = 1 << a.lpr_log2;
+  const int lane_in_row = t & (lpr - 1);
+  const int rows_per_wg = kBlock >> a.lpr_log2;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (t >> a.lpr_log2);
+  if (n >= a.N) return;
+  const int quad_base = blockIdx.y * (lpr * SLOTS) + lane_in_row;
+
+  float sc, mnv;
+  if constexpr (BF16P) {
+    sc = bf16_to_f32(static_cast<const uint16_t*>(a.scale)[n]);
+    mnv = bf16_to_f32(static_cast<const uint16_t*>(a.mn)[n]);
+  } else {
+    sc = static_cast<const float*>(a.scale)[n];
+    mnv = static_cast<const float*>(a.mn)[n];
+  }
+  // One IEEE division per row instead of one per element: with rcp = RN(1/sc),
+  // exact_quotient() returns RN(q / sc) for every integer 0 <= q <= 255 as long
+  // as sc is a normal number far from the exponent limits; other rows divide.
+  const float asc = fabsf(sc);
+  const bool fast_div = asc >= 0x1p-64f && asc <= 0x1p64f;
+  const float rcp = 1.0f / sc;
+  const int shift = static_cast<int>(n & (WPT - 1)) * BITS;
+  const uint8_t* grp = a.packed + (n / WPT) * a.G;
+  float* orow = a.out + n * a.G;
+
+  uint32_t w[SLOTS];
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) {
+    const int c = quad_base + s * lpr;
+    w[s] = 0;
+    if (c < a.qpr) {
+      if (a.in_vec == 4) {
+        w[s] = *reinterpret_cast<const uint32_t*>(grp + 4 * c);
+      } else {
+        const int cnt = min(4, a.G - 4 * c);
+        for (int i = 0; i < cnt; ++i) w[s] |= static_cast<uint32_t>(grp[4 * c + i]) << (8 * i);
+      }
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) {
+    const int c = quad_base + s * lpr;
+    if (c >= a.qpr) continue;
+    const uint32_t f = (w[s] >> shift) & FIELD;
+    float r[4];
+    if (__builtin_expect(fast_div, 1)) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r[i] = exact_quotient(static_cast<float>((f >> (8 * i)) & 0xFFu), sc, rcp) + mnv;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        // quantization_cuda_kernel.cu:182: true division, then add
+        r[i] = static_cast<float>((f >> (8 * i)) & 0xFFu) / sc + mnv;
+      }
+    }
+    store_quad<VEC>(orow + 4 * c, min(4, a.G - 4 * c), r);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct UnpackGeometry {
+  int qpr, lpr_log2, grid_y;
+};
+
+// Lanes per row for rows of G columns, two quads per lane; rows longer than
+// 64 lanes' worth are tiled over grid.y.
+static UnpackGeometry plan_unpack(int64_t G) {
+  UnpackGeometry g;
+  g.qpr = static_cast<int>((G + 3) / 4);
+  const int lanes_needed = (g.qpr + 1) / 2;
+  int l2 = 1;
+  while ((1 << l2) < lanes_needed && l2 < 5) ++l2;
+  g.lpr_log2 = l2;
+  const int quads_per_pass = (1 << l2) * 2;
+  g.grid_y = (g.qpr + quads_per_pass - 1) / quads_per_pass;
+  return g;
+}
+
+static bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+template <int BITS, bool BF16P>
+static void launch_unpack_variant(const UnpackArgs& a, bool vec4, dim3 grid, hipStream_t s) {
+  if (vec4)
+    hipLaunchKernelGGL((unpack_kernel<BITS, 2, 4, BF16P>), grid, dim3(kBlock), 0, s, a);
+  else
+    hipLaunchKernelGGL((unpack_kernel<BITS, 2, 1, BF16P>), grid, dim3(kBlock), 0, s, a);
+}
+
+template <bool BF16P>
+static int unpack_common(const uint8_t* packed, int bits, const void* scale, const void* mn,
+                         int64_t N, int64_t G, float* out, hipStream_t s) {
+  if (bits != 1 && bits != 2 && bits != 4 && bits != 8) return EXACT_E_BITS;
+  if (N < 0 || G < 0 || N > 0xFFFFFFFFll || G > 0x7FFFFFF0ll) return EXACT_E_SHAPE;
+  if (N == 0 || G == 0) return EXACT_OK;
+  if (!packed || !scale || !mn || !out) return EXACT_E_NULL;
+  const UnpackGeometry g = plan_unpack(G);
+  UnpackArgs a;
+  a.packed = packed;
+  a.scale = scale;
+  a.mn = mn;
+  a.N = N;
+  a.G = static_cast<int>(G);
+  a.qpr = g.qpr;
+  a.lpr_log2 = g.lpr_log2;
+  a.out = out;
+  a.in_vec = (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
+  const bool vec4 = (G % 4 == 0) && aligned(out, 16);
+  const int rows_per_wg = kBlock >> g.lpr_log2;
+  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(g.grid_y));
+  switch (bits) {
+    case 1: launch_unpack_variant<1, BF16P>(a, vec4, grid, s); break;
+    case 2: launch_unpack_variant<2, BF16P>(a, vec4, grid, s); break;
+    case 4: launch_unpack_variant<4, BF16P>(a, vec4, grid, s); break;
+    default: launch_unpack_variant<8, BF16P>(a, vec4, grid, s); break;
+  }
+  return launch_status();
+}
+
+}  // namespace exact
+
+using namespace exact;
+
+extern "C" {
+
+int exact_unpack_f32(const uint8_t* packed, int bits, const float* scale, const float* mn, int64_t N,
+                     int64_t G, float* out, void* stream) {
+  return unpack_common<false>(packed, bits, scale, mn, N, G, out, static_cast<hipStream_t>(stream));
+}
+
+int exact_unpack_bf16param_f32(const uint8_t* packed, int bits, const uint16_t* scale_bf16,
+                               const uint16_t* min_bf16, int64_t N, int64_t G, float* out, void* stream) {
+  return unpack_common<true>(packed, bits, scale_bf16, min_bf16, N, G, out, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -45,7 +45,7 @@ template <int VEC, int NT>
 __global__ __launch_bounds__(kBlock) void rp_fwd_kernel(const float* __restrict__ X,
                                                         const float* __restrict__ R, int64_t N, int D,
                                                         int k, float* __restrict__ out) {
-  extern __shared__ float Rl[];  // [kFwdDChunk][NT * 32]
+  HIP_DYNAMIC_SHARED(float, Rl)  // [kFwdDChunk][NT * 32]
   constexpr int KP = NT * kTile;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
@@ -100,7 +100,7 @@ template <int VEC, int NT>
 __global__ __launch_bounds__(kBlock) void rp_bwd_kernel(const float* __restrict__ Xr,
                                                         const float* __restrict__ R, int64_t N, int D,
                                                         int k, int kpad, float* __restrict__ out) {
-  extern __shared__ float Rl[];  // [NT * 32][kpad + 1], odd pitch: conflict-free column reads
+  HIP_DYNAMIC_SHARED(float, Rl)  // [NT * 32][kpad + 1], odd pitch: conflict-free column reads
   const int pitch = kpad + 1;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;

@@ -151,9 +151,9 @@ __global__ __launch_bounds__(kBlock) void spmm_chunk_kernel(const I* __restrict_
     for (int u = 0; u < kGather; ++u) {
 #pragma unroll
       for (int c = 0; c < VEC; ++c) xv[u][c] = 0.f;
-      if (base + u < cnt && kok) {
+      if (base + u < cnt) {  // wave-uniform, so every lane takes part in the broadcast
         const int64_t c = readlane_i(my_col, base + u);
-        load_vec<VEC>(X + c * K + kcol, xv[u]);
+        if (kok) load_vec<VEC>(X + c * K + kcol, xv[u]);
       }
     }
 #pragma unroll

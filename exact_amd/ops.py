@@ -19,7 +19,8 @@ from .conf import config
 from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import quantization as ext_quantization
 from .cpp_extension import spmm
-from .cpp_extension._checks import check_device_tensor, ptr, stream_ptr
+from .cpp_extension import _checks
+from .cpp_extension._checks import check_device_tensor, ptr
 from .utils import empty_cache, swap_to_cpu
 
 
@@ -138,7 +139,7 @@ def input2rp(input, kept_acts):  # noqa: A002
     N, D = input.shape
     rand_matrix = _gen_rand_matrix(D, kept_acts, input.device, input.dtype).contiguous()
     out = torch.empty((N, kept_acts), dtype=input.dtype, device=input.device)
-    rc = _lib.lib().exact_rp_fwd_f32(ptr(input), ptr(rand_matrix), N, D, kept_acts, ptr(out), stream_ptr(input))
+    rc = _lib.lib().exact_rp_fwd_f32(ptr(input), ptr(rand_matrix), N, D, kept_acts, ptr(out), _checks.stream_ptr(input))
     _lib.check(rc, "input2rp")
     return out, rand_matrix
 
@@ -155,7 +156,7 @@ def rp2input(dim_reduced_input, input_shape, rand_matrix):
         raise RuntimeError("rand_matrix does not match the reduced input")
     out = torch.empty((N, D), dtype=dim_reduced_input.dtype, device=dim_reduced_input.device)
     rc = _lib.lib().exact_rp_bwd_f32(ptr(dim_reduced_input), ptr(rand_matrix), N, D, k, ptr(out),
-                                     stream_ptr(dim_reduced_input))
+                                     _checks.stream_ptr(dim_reduced_input))
     _lib.check(rc, "rp2input")
     return out.view(input_shape)
 

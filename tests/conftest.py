@@ -31,3 +31,35 @@ def _reset_config():
     yield
     config.__dict__.clear()
     config.__dict__.update(saved)
+
+
+def _use_emulated_backend(monkeypatch):
+    """Run the Python layers on CPU tensors against the SIMT-emulated build of
+    the kernels (tests/emu): same .hip sources, same C ABI.  Only tests do
+    this; the package itself has no CPU path."""
+    import itertools
+
+    import torch
+
+    import emu_util
+    from exact_amd import _lib
+    from exact_amd.cpp_extension import _checks, quantization
+
+    monkeypatch.setattr(_lib, "_lib", emu_util.emu())
+    monkeypatch.setattr(_checks, "on_device", lambda t: True)
+    monkeypatch.setattr(_checks, "stream_ptr", lambda t: None)
+    counter = itertools.count(1)
+    monkeypatch.setattr(quantization, "next_philox", lambda device: (0xC0FFEE, 4 * next(counter)))
+    return torch.device("cpu")
+
+
+@pytest.fixture(params=["emulated", pytest.param("gpu", marks=pytest.mark.gpu)])
+def backend(request, monkeypatch):
+    """Device on which a layer-level test runs: the real GPU (marked gpu) or
+    CPU tensors over the emulated kernels."""
+    import torch
+    if request.param == "gpu":
+        if not torch.cuda.is_available():
+            pytest.skip("no GPU")
+        return torch.device("cuda:0")
+    return _use_emulated_backend(monkeypatch)

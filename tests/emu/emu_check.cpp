@@ -1,0 +1,217 @@
+// AddressSanitizer driver for the SIMT-emulated kernels (TESTS ONLY).
+//
+// Calls every C-ABI entry point on heap buffers of EXACTLY the documented
+// sizes, so that any out-of-bounds load or store of a kernel is reported by
+// ASan, and compares the results with the C oracle.  Usage:
+//     emu_check [quick|full]
+// `full` adds the benchmark shapes (169343 x 256 and a 169343-node graph).
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "../../include/exact_hip.h"
+
+extern "C" {
+void oracle_row_minmax(const float*, int64_t, int64_t, float*, float*);
+void oracle_scale(const float*, const float*, int64_t, int, float*);
+void oracle_pack(const float*, const float*, const float*, const float*, uint64_t, uint64_t, int64_t, int64_t, int,
+                 uint8_t*);
+void oracle_unpack(const uint8_t*, int, const float*, const float*, int64_t, int64_t, float*);
+uint16_t oracle_f32_to_bf16(float);
+void oracle_relu_fwd(const float*, int64_t, float*, uint32_t*);
+void oracle_relu_bwd(const float*, const uint32_t*, int64_t, float*);
+void oracle_dropout_fwd(const float*, const float*, uint64_t, uint64_t, float, int64_t, float*, uint32_t*);
+void oracle_dropout_bwd(const float*, const uint32_t*, float, int64_t, float*);
+void oracle_spmm_csr(const int64_t*, const int64_t*, const float*, const float*, int64_t, int64_t, int, float*);
+void oracle_rp_fwd(const float*, const float*, int64_t, int64_t, int64_t, float*);
+void oracle_rp_bwd(const float*, const float*, int64_t, int64_t, int64_t, float*);
+}
+
+static int g_fail = 0;
+#define CHECK(cond, ...)                                   \
+  do {                                                     \
+    if (!(cond)) {                                         \
+      std::fprintf(stderr, "FAIL %s:%d: ", __FILE__, __LINE__); \
+      std::fprintf(stderr, __VA_ARGS__);                   \
+      std::fprintf(stderr, "\n");                          \
+      ++g_fail;                                            \
+    }                                                      \
+  } while (0)
+
+// malloc'd, exactly sized: ASan puts red zones right behind the last element
+template <typename T>
+struct Buf {
+  T* p;
+  size_t n;
+  explicit Buf(size_t n_) : p(static_cast<T*>(std::malloc(n_ ? n_ * sizeof(T) : 1))), n(n_) {}
+  ~Buf() { std::free(p); }
+  T& operator[](size_t i) { return p[i]; }
+};
+
+static void check_quant(int64_t N, int64_t G, int bits, bool supplied, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 2.f);
+  std::uniform_real_distribution<float> ud(0.f, 1.f);
+  Buf<float> x(N * G), u(N * G), mn(N), mx(N), sc(N), mn2(N), sc2(N), out(N * G), want_out(N * G);
+  for (int64_t i = 0; i < N * G; ++i) { x[i] = nd(rng); u[i] = ud(rng); if (u[i] >= 1.f) u[i] = 0.5f; }
+  const int64_t nb = exact_packed_nbytes(N, G, bits);
+  Buf<uint8_t> packed(nb), want(nb), packed2(nb);
+  Buf<uint16_t> sbf(N), mbf(N);
+  const uint64_t seed = 0x1234abcd5678ull, off = (5ull << 32) + 17;
+  oracle_row_minmax(x.p, N, G, mn.p, mx.p);
+  oracle_scale(mn.p, mx.p, N, bits, sc.p);
+  std::memset(want.p, 0, nb);
+  oracle_pack(x.p, mn.p, sc.p, supplied ? u.p : nullptr, seed, off, N, G, bits, want.p);
+  int rc = exact_minmax_pack_f32(x.p, supplied ? u.p : nullptr, seed, off, N, G, bits, packed.p, sc2.p, mn2.p, sbf.p,
+                                 mbf.p, nullptr);
+  CHECK(rc == 0, "minmax_pack rc=%d", rc);
+  CHECK(std::memcmp(packed.p, want.p, nb) == 0, "packed bytes differ N=%ld G=%ld bits=%d supplied=%d", (long)N, (long)G, bits, supplied);
+  CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "scale/min differ N=%ld G=%ld", (long)N, (long)G);
+  rc = exact_pack_f32(x.p, mn.p, sc.p, supplied ? u.p : nullptr, seed, off, N, G, bits, packed2.p, nullptr);
+  CHECK(rc == 0 && std::memcmp(packed2.p, want.p, nb) == 0, "two-step pack differs N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  // unpack with bf16 parameters
+  Buf<float> scw(N), mnw(N);
+  for (int64_t n = 0; n < N; ++n) {
+    CHECK(sbf[n] == oracle_f32_to_bf16(sc[n]) && mbf[n] == oracle_f32_to_bf16(mn[n]), "bf16 params differ row %ld", (long)n);
+    uint32_t a = (uint32_t)sbf[n] << 16, b = (uint32_t)mbf[n] << 16;
+    std::memcpy(&scw[n], &a, 4);
+    std::memcpy(&mnw[n], &b, 4);
+  }
+  oracle_unpack(want.p, bits, scw.p, mnw.p, N, G, want_out.p);
+  rc = exact_unpack_bf16param_f32(packed.p, bits, sbf.p, mbf.p, N, G, out.p, nullptr);
+  CHECK(rc == 0 && std::memcmp(out.p, want_out.p, N * G * 4) == 0, "unpack(bf16) differs N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  oracle_unpack(want.p, bits, sc.p, mn.p, N, G, want_out.p);
+  rc = exact_unpack_f32(packed.p, bits, sc.p, mn.p, N, G, out.p, nullptr);
+  CHECK(rc == 0 && std::memcmp(out.p, want_out.p, N * G * 4) == 0, "unpack(f32) differs N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  Buf<float> rmn(N), rmx(N);
+  rc = exact_row_minmax_f32(x.p, N, G, rmn.p, rmx.p, nullptr);
+  CHECK(rc == 0 && std::memcmp(rmn.p, mn.p, N * 4) == 0 && std::memcmp(rmx.p, mx.p, N * 4) == 0, "row_minmax differs");
+}
+
+static void check_masks(int64_t n, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 1.f);
+  std::uniform_real_distribution<float> ud(0.f, 1.f);
+  const int64_t words = (n + 31) / 32;
+  Buf<float> x(n), u(n), g(n), y(n), wy(n), dx(n), wdx(n);
+  Buf<uint32_t> m(words), wm(words);
+  for (int64_t i = 0; i < n; ++i) { x[i] = nd(rng); u[i] = ud(rng); g[i] = nd(rng); }
+  oracle_relu_fwd(x.p, n, wy.p, wm.p);
+  CHECK(exact_relu_fwd_f32(x.p, n, y.p, m.p, nullptr) == 0, "relu rc");
+  CHECK(std::memcmp(y.p, wy.p, n * 4) == 0 && std::memcmp(m.p, wm.p, words * 4) == 0, "relu fwd differs n=%ld", (long)n);
+  oracle_relu_bwd(g.p, wm.p, n, wdx.p);
+  CHECK(exact_relu_bwd_f32(g.p, m.p, n, dx.p, nullptr) == 0 && std::memcmp(dx.p, wdx.p, n * 4) == 0, "relu bwd differs n=%ld", (long)n);
+  for (int mode = 0; mode < 2; ++mode) {
+    const float p = mode ? 0.1f : 0.5f;
+    const float* noise = mode ? nullptr : u.p;
+    oracle_dropout_fwd(x.p, noise, 99, 7, p, n, wy.p, wm.p);
+    CHECK(exact_dropout_fwd_f32(x.p, noise, 99, 7, p, n, y.p, m.p, nullptr) == 0, "dropout rc");
+    CHECK(std::memcmp(y.p, wy.p, n * 4) == 0 && std::memcmp(m.p, wm.p, words * 4) == 0, "dropout fwd differs n=%ld mode=%d", (long)n, mode);
+    oracle_dropout_bwd(g.p, wm.p, p, n, wdx.p);
+    CHECK(exact_dropout_bwd_f32(g.p, m.p, p, n, dx.p, nullptr) == 0 && std::memcmp(dx.p, wdx.p, n * 4) == 0, "dropout bwd differs n=%ld", (long)n);
+  }
+}
+
+struct Csr {
+  std::vector<int64_t> rowptr, col;
+  std::vector<float> val;
+};
+
+static Csr powerlaw(int64_t M, int64_t ncols, double avg, int64_t hub, std::mt19937& rng) {
+  Csr g;
+  g.rowptr.assign(M + 1, 0);
+  std::uniform_real_distribution<double> ud(0.0, 1.0);
+  std::normal_distribution<float> nd(0.f, 1.f);
+  for (int64_t r = 0; r < M; ++r) {
+    // Pareto-tailed degree with the requested mean-ish, some empty rows
+    double d = avg * 0.5 / std::pow(1.0 - ud(rng), 1.0 / 1.3);
+    int64_t deg = ud(rng) < 0.02 ? 0 : std::min<int64_t>((int64_t)d, ncols);
+    if (hub && (r == M / 3 || r == M / 2)) deg = std::min(hub, ncols);
+    g.rowptr[r + 1] = g.rowptr[r] + deg;
+    for (int64_t i = 0; i < deg; ++i) {
+      g.col.push_back((int64_t)(ud(rng) * ncols) % ncols);
+      g.val.push_back(nd(rng));
+    }
+  }
+  return g;
+}
+
+static void check_spmm(int64_t M, int64_t ncols, int64_t K, double avg, int64_t hub, std::mt19937& rng) {
+  const Csr g = powerlaw(M, ncols, avg, hub, rng);
+  const int64_t nnz = (int64_t)g.col.size();
+  std::normal_distribution<float> nd(0.f, 1.f);
+  Buf<float> X(ncols * K), out(M * K), want(M * K), val(nnz);
+  Buf<int64_t> rp64(M + 1), col64(nnz);
+  Buf<int32_t> rp32(M + 1), col32(nnz);
+  for (int64_t i = 0; i < ncols * K; ++i) X[i] = nd(rng);
+  for (int64_t i = 0; i <= M; ++i) { rp64[i] = g.rowptr[i]; rp32[i] = (int32_t)g.rowptr[i]; }
+  for (int64_t i = 0; i < nnz; ++i) { col64[i] = g.col[i]; col32[i] = (int32_t)g.col[i]; val[i] = g.val[i]; }
+  for (int reduce = 0; reduce < 2; ++reduce)
+    for (int valued = 0; valued < 2; ++valued)
+      for (int wide = 0; wide < 2; ++wide) {
+        oracle_spmm_csr(rp64.p, col64.p, valued ? val.p : nullptr, X.p, M, K, reduce, want.p);
+        const int rc = wide ? exact_spmm_csr_f32(rp64.p, col64.p, valued ? val.p : nullptr, 8, X.p, M, ncols, K, nnz, reduce, out.p, nullptr)
+                            : exact_spmm_csr_f32(rp32.p, col32.p, valued ? val.p : nullptr, 4, X.p, M, ncols, K, nnz, reduce, out.p, nullptr);
+        CHECK(rc == 0, "spmm rc=%d", rc);
+        double worst = 0, scale = 1e-30;
+        for (int64_t i = 0; i < M * K; ++i) scale = std::max(scale, (double)std::fabs(want[i]));
+        for (int64_t i = 0; i < M * K; ++i) worst = std::max(worst, (double)std::fabs(out[i] - want[i]));
+        CHECK(worst <= 1e-5 * scale, "spmm differs M=%ld K=%ld reduce=%d valued=%d wide=%d: %g of %g", (long)M, (long)K, reduce, valued, wide, worst, scale);
+      }
+}
+
+static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 1.f);
+  Buf<float> X(N * D), R(D * k), xr(N * k), wxr(N * k), back(N * D), wback(N * D);
+  for (int64_t i = 0; i < N * D; ++i) X[i] = nd(rng);
+  for (int64_t i = 0; i < D * k; ++i) R[i] = nd(rng) / std::sqrt((float)k);
+  oracle_rp_fwd(X.p, R.p, N, D, k, wxr.p);
+  CHECK(exact_rp_fwd_f32(X.p, R.p, N, D, k, xr.p, nullptr) == 0, "rp fwd rc");
+  double worst = 0, scale = 1e-30;
+  for (int64_t i = 0; i < N * k; ++i) { scale = std::max(scale, (double)std::fabs(wxr[i])); worst = std::max(worst, (double)std::fabs(xr[i] - wxr[i])); }
+  CHECK(worst <= 2e-5 * scale, "rp fwd differs N=%ld D=%ld k=%ld: %g of %g", (long)N, (long)D, (long)k, worst, scale);
+  oracle_rp_bwd(wxr.p, R.p, N, D, k, wback.p);
+  CHECK(exact_rp_bwd_f32(wxr.p, R.p, N, D, k, back.p, nullptr) == 0, "rp bwd rc");
+  worst = 0, scale = 1e-30;
+  for (int64_t i = 0; i < N * D; ++i) { scale = std::max(scale, (double)std::fabs(wback[i])); worst = std::max(worst, (double)std::fabs(back[i] - wback[i])); }
+  CHECK(worst <= 2e-5 * scale, "rp bwd differs N=%ld D=%ld k=%ld: %g of %g", (long)N, (long)D, (long)k, worst, scale);
+}
+
+int main(int argc, char** argv) {
+  const std::string mode = argc > 1 ? argv[1] : "quick";
+  std::mt19937 rng(12345);
+  const int64_t shapes[][2] = {{1, 1}, {5, 3}, {37, 25}, {64, 32}, {100, 76}, {33, 40}, {129, 100}, {300, 128},
+                               {203, 256}, {61, 602}, {16, 1024}, {19, 520}, {9, 1500}, {7, 2048}, {8, 8}, {3, 4}};
+  for (auto& s : shapes)
+    for (int bits : {1, 2, 4, 8})
+      for (int supplied = 0; supplied < 2; ++supplied) check_quant(s[0], s[1], bits, supplied, rng);
+  std::printf("quant shapes ok (failures so far %d)\n", g_fail);
+  for (int64_t n : {1, 3, 4, 7, 8, 31, 32, 33, 255, 256, 257, 1000, 2048, 2049, 4101, 50001}) check_masks(n, rng);
+  std::printf("mask sizes ok (failures so far %d)\n", g_fail);
+  check_spmm(300, 300, 256, 8, 200, rng);
+  check_spmm(200, 200, 40, 5, 0, rng);
+  check_spmm(100, 100, 602, 10, 90, rng);
+  check_spmm(500, 77, 100, 10, 0, rng);
+  check_spmm(64, 64, 1, 3, 0, rng);
+  check_spmm(90, 90, 47, 4, 80, rng);
+  check_spmm(130, 130, 6, 30, 120, rng);
+  check_spmm(4, 9, 8, 0, 0, rng);
+  std::printf("spmm shapes ok (failures so far %d)\n", g_fail);
+  const int64_t rps[][3] = {{1, 256, 32}, {31, 256, 32}, {200, 256, 32}, {130, 602, 76}, {140, 100, 25}, {129, 256, 64},
+                            {64, 128, 64}, {77, 50, 15}, {130, 7, 4}, {100, 256, 126}, {33, 256, 128}};
+  for (auto& s : rps) check_rp(s[0], s[1], s[2], rng);
+  std::printf("rp shapes ok (failures so far %d)\n", g_fail);
+  if (mode == "full") {
+    for (int bits : {1, 2, 4, 8}) check_quant(169343, 256, bits, bits == 2, rng);
+    std::printf("full-size quant ok (failures so far %d)\n", g_fail);
+    check_masks(169343ll * 256, rng);
+    check_spmm(169343, 169343, 256, 14, 20000, rng);
+    check_spmm(169343, 169343, 40, 14, 20000, rng);
+    check_rp(169343, 256, 32, rng);
+    std::printf("full-size spmm/rp/masks ok (failures so far %d)\n", g_fail);
+  }
+  std::printf(g_fail ? "FAILED: %d check(s)\n" : "all checks passed\n", g_fail);
+  return g_fail ? 1 : 0;
+}

@@ -1,0 +1,167 @@
+"""Load the SIMT-emulated build of the kernels (tests/emu) and call its C ABI
+with NumPy arrays.  The emulated library is compiled from the very same .hip
+sources as libexact_hip.so; it exists so that the kernels' indexing and
+arithmetic are checked on machines without a GPU."""
+import ctypes
+import importlib.util
+import os
+
+import numpy as np
+
+from exact_amd import _lib
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_spec = importlib.util.spec_from_file_location("build_emu", os.path.join(HERE, "emu", "build_emu.py"))
+build_emu = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(build_emu)
+
+_emu = None
+
+
+def _newest_source_mtime():
+    files = [os.path.join(build_emu.CSRC, f) for f in os.listdir(build_emu.CSRC) if f.endswith((".hip", ".hpp"))]
+    files.append(os.path.join(HERE, "emu", "include", "hip", "hip_runtime.h"))
+    return max(os.path.getmtime(f) for f in files)
+
+
+def emu():
+    global _emu
+    if _emu is None:
+        if not os.path.exists(build_emu.LIB) or os.path.getmtime(build_emu.LIB) < _newest_source_mtime():
+            build_emu.build_lib()
+        handle = ctypes.CDLL(build_emu.LIB)
+        for name, (res, args) in _lib.SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _emu = handle
+    return _emu
+
+
+def p(a):
+    return None if a is None else a.ctypes.data
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def minmax_pack(x, bits, noise=None, seed=0, offset=0, guard=64):
+    """-> (packed u8, scale f32, min f32, scale bf16 bits, min bf16 bits); the
+    packed buffer has `guard` sentinel bytes behind it that must stay intact."""
+    x = f32(x)
+    N, G = x.shape
+    nb = int(emu().exact_packed_nbytes(N, G, bits))
+    packed = np.full(nb + guard, 0xA5, np.uint8)
+    s32, m32 = np.zeros(N, np.float32), np.zeros(N, np.float32)
+    sbf, mbf = np.zeros(N, np.uint16), np.zeros(N, np.uint16)
+    noise = None if noise is None else f32(noise)
+    rc = emu().exact_minmax_pack_f32(p(x), p(noise), seed, offset, N, G, bits, p(packed), p(s32), p(m32), p(sbf),
+                                     p(mbf), None)
+    assert rc == 0, rc
+    assert (packed[nb:] == 0xA5).all(), "pack wrote past the packed stream"
+    return packed[:nb], s32, m32, sbf, mbf
+
+
+def pack(x, mn, scale, bits, noise=None, seed=0, offset=0, guard=64):
+    x = f32(x)
+    N, G = x.shape
+    nb = int(emu().exact_packed_nbytes(N, G, bits))
+    packed = np.full(nb + guard, 0xA5, np.uint8)
+    noise = None if noise is None else f32(noise)
+    rc = emu().exact_pack_f32(p(x), p(f32(mn)), p(f32(scale)), p(noise), seed, offset, N, G, bits, p(packed), None)
+    assert rc == 0, rc
+    assert (packed[nb:] == 0xA5).all()
+    return packed[:nb]
+
+
+def unpack(packed, bits, scale, mn, N, G, bf16=False, guard=64):
+    out = np.full(N * G + guard, np.float32(-12345.0), np.float32)
+    packed = np.ascontiguousarray(packed)
+    if bf16:
+        rc = emu().exact_unpack_bf16param_f32(p(packed), bits, p(np.ascontiguousarray(scale, np.uint16)),
+                                              p(np.ascontiguousarray(mn, np.uint16)), N, G, p(out), None)
+    else:
+        rc = emu().exact_unpack_f32(p(packed), bits, p(f32(scale)), p(f32(mn)), N, G, p(out), None)
+    assert rc == 0, rc
+    assert (out[N * G:] == np.float32(-12345.0)).all(), "unpack wrote past the output"
+    return out[:N * G].reshape(N, G)
+
+
+def row_minmax(x):
+    x = f32(x)
+    N, G = x.shape
+    mn, mx = np.zeros(N, np.float32), np.zeros(N, np.float32)
+    assert emu().exact_row_minmax_f32(p(x), N, G, p(mn), p(mx), None) == 0
+    return mn, mx
+
+
+def relu_fwd(x, guard=8):
+    x = f32(x).reshape(-1)
+    n = x.size
+    y = np.full(n + guard, np.float32(7.0), np.float32)
+    words = (n + 31) // 32
+    mask = np.full(words + guard, 0x5A5A5A5A, np.uint32)
+    assert emu().exact_relu_fwd_f32(p(x), n, p(y), p(mask), None) == 0
+    assert (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
+    return y[:n], mask[:words]
+
+
+def relu_bwd(dy, mask):
+    dy = f32(dy).reshape(-1)
+    dx = np.zeros_like(dy)
+    assert emu().exact_relu_bwd_f32(p(dy), p(np.ascontiguousarray(mask, np.uint32)), dy.size, p(dx), None) == 0
+    return dx
+
+
+def dropout_fwd(x, prob, noise=None, seed=0, offset=0, guard=8):
+    x = f32(x).reshape(-1)
+    n = x.size
+    y = np.full(n + guard, np.float32(7.0), np.float32)
+    words = (n + 31) // 32
+    mask = np.full(words + guard, 0x5A5A5A5A, np.uint32)
+    noise = None if noise is None else f32(noise).reshape(-1)
+    assert emu().exact_dropout_fwd_f32(p(x), p(noise), seed, offset, prob, n, p(y), p(mask), None) == 0
+    assert (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
+    return y[:n], mask[:words]
+
+
+def dropout_bwd(dy, mask, prob):
+    dy = f32(dy).reshape(-1)
+    dx = np.zeros_like(dy)
+    assert emu().exact_dropout_bwd_f32(p(dy), p(np.ascontiguousarray(mask, np.uint32)), prob, dy.size, p(dx), None) == 0
+    return dx
+
+
+def spmm(rowptr, col, val, X, reduce, idx=np.int64, guard=16):
+    rowptr = np.ascontiguousarray(rowptr, dtype=idx)
+    col = np.ascontiguousarray(col, dtype=idx)
+    X = f32(X)
+    val = None if val is None else f32(val)
+    M, K = rowptr.size - 1, X.shape[1]
+    out = np.full(M * K + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_spmm_csr_f32(p(rowptr), p(col), p(val), rowptr.itemsize, p(X), M, X.shape[0], K, col.size,
+                                  1 if reduce == "mean" else 0, p(out), None)
+    assert rc == 0, rc
+    assert (out[M * K:] == np.float32(-777.0)).all()
+    return out[:M * K].reshape(M, K)
+
+
+def rp_fwd(X, R, guard=16):
+    X, R = f32(X), f32(R)
+    N, D = X.shape
+    k = R.shape[1]
+    out = np.full(N * k + guard, np.float32(-777.0), np.float32)
+    assert emu().exact_rp_fwd_f32(p(X), p(R), N, D, k, p(out), None) == 0
+    assert (out[N * k:] == np.float32(-777.0)).all()
+    return out[:N * k].reshape(N, k)
+
+
+def rp_bwd(Xr, R, guard=16):
+    Xr, R = f32(Xr), f32(R)
+    N, k = Xr.shape
+    D = R.shape[0]
+    out = np.full(N * D + guard, np.float32(-777.0), np.float32)
+    assert emu().exact_rp_bwd_f32(p(Xr), p(R), N, D, k, p(out), None) == 0
+    assert (out[N * D:] == np.float32(-777.0)).all()
+    return out[:N * D].reshape(N, D)

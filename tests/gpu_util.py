@@ -39,3 +39,33 @@ def bytes_equal(t, arr):
         t = t.view(torch.int16)
     a = t.numpy()
     return np.array_equal(a.view(np.uint8).reshape(-1), np.ascontiguousarray(arr).view(np.uint8).reshape(-1))
+
+
+class SeededNoise:
+    """Uniform [0, 1) noise (and projection matrices) that depends only on
+    (seed, call index, shape): the product and the oracle model each hold one
+    and, making their draws in the same order, see identical bits."""
+
+    def __init__(self, seed):
+        self.seed, self.calls = seed, 0
+
+    def _gen(self):
+        self.calls += 1
+        return torch.Generator().manual_seed(self.seed * 1000003 + self.calls)
+
+    def noise(self, shape, device=None):
+        n = int(np.prod(shape))
+        t = torch.rand(n, generator=self._gen(), dtype=torch.float32).view(*shape) if n else torch.zeros(shape)
+        return t if device is None else t.to(device)
+
+    def rademacher(self, D, k, device=None):
+        bern = torch.randint(2, (D, k), generator=self._gen()).float()
+        R = (2.0 * bern - 1) / k ** 0.5
+        return R if device is None else R.to(device)
+
+    # the two callables exact_amd.config expects
+    def noise_source(self, shape, device):
+        return self.noise(tuple(shape), device)
+
+    def rp_matrix_source(self, D, k, device):
+        return self.rademacher(D, k, device)

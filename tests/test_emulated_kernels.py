@@ -1,0 +1,138 @@
+"""The library's .hip kernels, compiled unchanged for a CPU SIMT emulator
+(tests/emu), checked against the oracle: same parity bar as the GPU tests
+(bit-exact for bytes, masks and dequantised values; 1e-5 relative for SpMM and
+the projection GEMMs), plus sentinel bytes behind every output buffer.  This
+is what verifies kernel indexing and arithmetic when no GPU is at hand; the
+GPU tests (-m gpu) remain the parity tests proper."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+import emu_util as e
+import exact_oracle as o
+
+F32 = np.float32
+SHAPES = [(1, 1), (5, 3), (37, 25), (64, 32), (100, 76), (33, 40), (129, 100), (300, 128), (200, 256),
+          (61, 602), (16, 1024), (19, 520), (9, 1500), (7, 2048), (8, 8), (24, 16), (3, 4)]
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("N,G", SHAPES)
+def test_pack_unpack(bits, N, G):
+    rng = np.random.default_rng(N * 7 + G + bits)
+    x = (rng.standard_normal((N, G)) * 3).astype(F32)
+    if N > 4:
+        x[2] = 0.75                                          # a constant row
+    u = rng.random((N, G), dtype=F32)
+    want = o.quantize_activation(x, bits, u)
+    packed, s32, m32, sbf, mbf = e.minmax_pack(x, bits, u)
+    assert np.array_equal(packed, want[0])
+    assert np.array_equal(s32.view(np.uint32), want[4].view(np.uint32)) and np.array_equal(m32, want[5])
+    assert np.array_equal(sbf, want[2]) and np.array_equal(mbf, want[3])
+    xh = e.unpack(packed, bits, sbf, mbf, N, G, bf16=True)
+    assert np.array_equal(xh.view(np.uint32), o.dequantize_activation(want[0], bits, want[2], want[3], (N, G)).view(np.uint32))
+    xh32 = e.unpack(packed, bits, s32, m32, N, G)
+    assert np.array_equal(xh32.view(np.uint32), o.unpack_single_precision(want[0], bits, want[4], want[5], N, G).view(np.uint32))
+    # two-step form and the stand-alone row statistics
+    mn, mx = e.row_minmax(x)
+    assert np.array_equal(mn, want[5]) and np.array_equal(mx, x.max(1))
+    assert np.array_equal(e.pack(x, mn, want[4], bits, u), want[0])
+    # internal Philox noise == oracle fed with the documented stream
+    seed, off = 0xABCDEF0123456789, (9 << 32) + 77
+    got = e.minmax_pack(x, bits, None, seed, off)[0]
+    assert np.array_equal(got, o.quantize_activation(x, bits, o.philox_noise_rows(seed, off, N, G))[0])
+    assert np.array_equal(e.pack(x, mn, want[4], bits, None, seed, off), got)
+
+
+def test_unpack_extreme_scales_take_the_division_path():
+    # scales outside [2^-64, 2^64], inf and nan rows use the per-element IEEE division
+    N, G, bits = 16, 24, 8
+    rng = np.random.default_rng(3)
+    packed = rng.integers(0, 256, o.packed_nbytes(N, G, bits), dtype=np.uint8)
+    scale = np.array([1e-30, 1e30, np.inf, 0.0, 3e-39, 1.5, 255.0 / 7, 1e25, 2.0 ** -64, 2.0 ** 64, 1e-20, 1e20,
+                      np.nan, -2.5, 1e38, 7e-5], F32)
+    mn = rng.standard_normal(N).astype(F32)
+    with np.errstate(all="ignore"):
+        want = o.unpack_single_precision(packed, bits, scale, mn, N, G)
+    got = e.unpack(packed, bits, scale, mn, N, G)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 7, 8, 31, 32, 33, 255, 256, 257, 1000, 2048, 2049, 4096 + 5, 50001])
+def test_relu_and_dropout(n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(F32)
+    x[: min(n, 3)] = [0.0, -0.0, np.nan][: min(n, 3)]
+    g = rng.standard_normal(n).astype(F32)
+    y, mask = e.relu_fwd(x)
+    wy, wm = o.relu_fwd(x)
+    assert np.array_equal(y.view(np.uint32), wy.view(np.uint32)) and np.array_equal(mask, wm)
+    assert np.array_equal(e.relu_bwd(g, mask), o.relu_bwd(g, wm))
+    u = rng.random(n, dtype=F32)
+    for p in (0.5, 0.1, 0.0, 0.9):
+        y, mask = e.dropout_fwd(x, p, u)
+        wy, wm = o.dropout_fwd(x, p, u)
+        assert np.array_equal(y.view(np.uint32), wy.view(np.uint32)) and np.array_equal(mask, wm)
+        assert np.array_equal(e.dropout_bwd(g, mask, p).view(np.uint32), o.dropout_bwd(g, wm, p).view(np.uint32))
+    seed, off = 1234567, (1 << 40) + 3
+    y, mask = e.dropout_fwd(x, 0.5, None, seed, off)
+    wy, wm = o.dropout_fwd(x, 0.5, o.philox_noise_flat(seed, off, n))
+    assert np.array_equal(y.view(np.uint32), wy.view(np.uint32)) and np.array_equal(mask, wm)
+
+
+def powerlaw_csr(M, avg_deg, seed, n_cols=None, hub=0):
+    rng = np.random.default_rng(seed)
+    n_cols = n_cols or M
+    deg = np.minimum((rng.zipf(2.1, M) * avg_deg / 2.5).astype(np.int64), n_cols)
+    deg[rng.integers(0, M, max(1, M // 50))] = 0
+    if hub:
+        deg[rng.integers(0, M, 3)] = min(hub, n_cols)
+    rows = np.repeat(np.arange(M), deg)
+    cols = rng.integers(0, n_cols, rows.size)
+    A = sp.coo_matrix((rng.standard_normal(rows.size).astype(F32), (rows, cols)), shape=(M, n_cols)).tocsr()
+    A.sum_duplicates()
+    A.sort_indices()
+    return A
+
+
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("valued", [True, False])
+@pytest.mark.parametrize("reduce", ["sum", "mean"])
+@pytest.mark.parametrize("M,K,avg,hub,ncols", [(300, 256, 8, 200, None), (200, 40, 5, 0, None), (100, 602, 10, 90, None),
+                                               (500, 100, 10, 0, 77), (64, 1, 3, 0, None), (90, 47, 4, 80, None),
+                                               (10, 128, 2, 0, None), (130, 6, 30, 120, None)])
+def test_spmm(M, K, avg, hub, ncols, reduce, valued, idx):
+    A = powerlaw_csr(M, avg, M + K, n_cols=ncols, hub=hub)
+    X = np.random.default_rng(K).standard_normal((A.shape[1], K)).astype(F32)
+    val = A.data if valued else None
+    want = o.spmm_csr(A.indptr, A.indices, val, X, reduce)
+    got = e.spmm(A.indptr, A.indices, val, X, reduce, idx)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * (np.abs(want).max() + 1e-30))
+    assert (got[np.diff(A.indptr) == 0] == 0).all()
+
+
+def test_spmm_all_empty_and_single_long_row():
+    X = np.ones((5, 8), F32)
+    z = e.spmm(np.zeros(5, np.int64), np.zeros(0, np.int64), None, X, "mean")
+    assert z.shape == (4, 8) and (z == 0).all()
+    rowptr = np.array([0, 0, 1000, 1000, 1003], np.int64)
+    col = np.random.default_rng(0).integers(0, 5, 1003)
+    got = e.spmm(rowptr, col, None, X, "sum")
+    assert np.array_equal(got[:, 0], np.array([0, 1000, 0, 3], F32))
+
+
+@pytest.mark.parametrize("dist", ["rademacher", "gaussian"])
+@pytest.mark.parametrize("N,D,frac", [(1, 256, 0.125), (31, 256, 0.125), (200, 256, 0.125), (130, 602, 0.125),
+                                      (140, 100, 0.25), (129, 256, 0.25), (64, 128, 0.5), (77, 50, 0.3), (130, 7, 0.5),
+                                      (100, 256, 0.49)])
+def test_rp(N, D, frac, dist):
+    k = o.kept_acts(frac, D)
+    rng = np.random.default_rng(N + D)
+    R = o.rademacher_matrix(D, k, rng) if dist == "rademacher" else o.gaussian_matrix(D, k, rng)
+    X = rng.standard_normal((N, D)).astype(F32)
+    want = o.input2rp(X, R)
+    got = e.rp_fwd(X, R)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+    back = e.rp_bwd(got, R)
+    wb = o.rp2input(got, R)
+    np.testing.assert_allclose(back, wb, rtol=1e-5, atol=1e-5 * np.abs(wb).max())

@@ -1,0 +1,259 @@
+"""Layer- and model-level parity: the quantised autograd Functions, the Q*
+layers and full training steps against the CPU oracle model
+(oracle/oracle_model.py), with the SAME noise / projection matrices on both
+sides.  Every test runs twice: on CPU tensors over the SIMT-emulated kernels
+(always) and on the GPU (-m gpu)."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import torch
+import torch.nn.functional as F
+
+import exact_amd as exact
+import oracle_model as om
+from exact_amd import ops
+from exact_amd.conf import config
+from exact_amd.models import GCN, SAGE
+from exact_amd.sparse import SparseTensor, gcn_norm
+from gpu_util import SeededNoise
+
+
+def tol(device):
+    # CPU tensors: both sides use the same torch CPU GEMMs; GPU: rocBLAS vs MKL
+    return dict(rtol=1e-5, atol=1e-6) if device.type == "cpu" else dict(rtol=2e-4, atol=2e-5)
+
+
+def wire_noise(seed):
+    a, b = SeededNoise(seed), SeededNoise(seed)
+    config.noise_source, config.rp_matrix_source = a.noise_source, a.rp_matrix_source
+    return b
+
+
+def er_graph(n, avg_deg, seed):
+    """Erdos-Renyi, symmetrised, as scipy CSR without values."""
+    rng = np.random.default_rng(seed)
+    m = int(n * avg_deg / 2)
+    r, c = rng.integers(0, n, m), rng.integers(0, n, m)
+    A = sp.coo_matrix((np.ones(2 * m, np.float32), (np.concatenate([r, c]), np.concatenate([c, r]))), shape=(n, n)).tocsr()
+    A.data[:] = 1.0
+    A.setdiag(0)
+    A.eliminate_zeros()
+    A.sort_indices()
+    return A
+
+
+@pytest.mark.parametrize("kept_frac,bits", [(1.0, 2), (0.25, 2), (0.125, 1), (1.0, 8)])
+def test_qlinear_matches_oracle(backend, kept_frac, bits):
+    config.kept_frac, config.activation_compression_bits = kept_frac, [bits]
+    other = wire_noise(11)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(300, 64, generator=g)
+    w = torch.randn(24, 64, generator=g) * 0.1
+    b = torch.randn(24, generator=g)
+    dy = torch.randn(300, 24, generator=g)
+    xd, wd, bd = (t.clone().to(backend).requires_grad_() for t in (x, w, b))
+    y = ops.qlinear.apply(xd, wd, bd, None, None, None, True)
+    y.backward(dy.to(backend))
+    xo, wo, bo = (t.clone().requires_grad_() for t in (x, w, b))
+    c = om.Ctx(bits, kept_frac, other.noise, other.rademacher)
+    yo = om.QLinearFn.apply(c, xo, wo, bo, None, None, None)
+    yo.backward(dy)
+    t = tol(backend)
+    torch.testing.assert_close(y.detach().cpu(), F.linear(x, w, b), **t)
+    torch.testing.assert_close(xd.grad.cpu(), xo.grad, **t)
+    torch.testing.assert_close(bd.grad.cpu(), bo.grad, **t)
+    torch.testing.assert_close(wd.grad.cpu(), wo.grad, rtol=1e-3, atol=1e-3)   # depends on the dequantised input
+    # and the weight gradient really is the one of the DEQUANTISED input, not of x
+    exact_gw = dy.t().mm(x)
+    assert (wd.grad.cpu() - exact_gw).abs().max() > 1e-3
+
+
+def test_quantised_linear_gradient_is_unbiased(backend):
+    """The reference only prints bias / std of repeated quantised backward
+    passes (test/test_op.py:297-330); here the bias must vanish as 1/sqrt(reps)."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(2000, 32, generator=g).to(backend)
+    w = (torch.randn(8, 32, generator=g) * 0.1).to(backend)
+    dy = torch.randn(2000, 8, generator=g).to(backend)
+    ref = dy.t().mm(x)
+    grads = []
+    for _ in range(24):
+        wd = w.clone().requires_grad_()
+        ops.qlinear.apply(x, wd, None, None, None, None, True).backward(dy)
+        grads.append(wd.grad)
+    grads = torch.stack(grads)
+    bias = (grads.mean(0) - ref).norm() / ref.norm()
+    single = (grads[0] - ref).norm() / ref.norm()
+    assert single > 0.02 and bias < single / 3
+
+
+def test_batch_norm_equals_stock_without_compression(backend):
+    """test/test_op.py:374-413: output and all three gradients within 1e-3."""
+    config.compress_activation = False
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(4000, 32, generator=g) * 0.01).to(backend)
+    dy = torch.randn(4000, 32, generator=g).to(backend)
+    bn, qbn = torch.nn.BatchNorm1d(32).to(backend), exact.QBatchNorm1d(32).to(backend)
+    outs = []
+    for layer in (bn, qbn):
+        xi = x.clone().requires_grad_()
+        y = layer(xi)
+        y.backward(dy)
+        outs.append((y.detach(), xi.grad, layer.weight.grad, layer.bias.grad, layer.running_mean, layer.running_var))
+    for a, b in zip(*outs):
+        torch.testing.assert_close(a, b, rtol=1e-3, atol=1e-3)
+
+
+def test_batch_norm_matches_oracle_with_compression(backend):
+    other = wire_noise(5)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(500, 16, generator=g)
+    dy = torch.randn(500, 16, generator=g)
+    qbn = exact.QBatchNorm1d(16).to(backend)
+    xi = x.clone().to(backend).requires_grad_()
+    y = qbn(xi)
+    y.backward(dy.to(backend))
+    xo = x.clone().requires_grad_()
+    wo, bo = torch.ones(16, requires_grad=True), torch.zeros(16, requires_grad=True)
+    c = om.Ctx(2, 1.0, other.noise, None)
+    yo = om.QBatchNormFn.apply(c, xo, torch.zeros(16), torch.ones(16), wo, bo, 0.1, 1e-5)
+    yo.backward(dy)
+    torch.testing.assert_close(y.detach().cpu(), yo.detach(), rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(xi.grad.cpu(), xo.grad, rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(qbn.weight.grad.cpu(), wo.grad, rtol=1e-3, atol=1e-3)
+    # eval mode is the stock layer
+    qbn.eval()
+    torch.testing.assert_close(qbn(x.to(backend)), F.batch_norm(x.to(backend), qbn.running_mean, qbn.running_var,
+                                                                qbn.weight, qbn.bias, False, 0.1, 1e-5))
+
+
+def test_relu_dropout_layers(backend):
+    x = torch.randn(100, 33, device=backend, requires_grad=True)
+    y = exact.QReLU()(x)
+    y.sum().backward()
+    assert torch.equal(y, F.relu(x)) and torch.equal(x.grad, (x > 0).float())
+    d = exact.QDropout(0.5)
+    xd = torch.ones(100, 33, device=backend, requires_grad=True)
+    yd = d(xd)
+    yd.sum().backward()
+    assert set(yd.unique().tolist()) <= {0.0, 2.0} and torch.equal(xd.grad, yd.detach())
+    d.eval()
+    assert torch.equal(d(xd), xd)
+    d2 = exact.QDropout2(0.5)
+    assert set(d2(xd).unique().tolist()) <= {0.0, 1.0}
+
+
+def _params_of_gcn(model):
+    m = model.model
+    return {"conv_w": [c.weight.detach().cpu().clone().requires_grad_() for c in m.convs],
+            "conv_b": [None if c.bias is None else c.bias.detach().cpu().clone().requires_grad_() for c in m.convs],
+            "bn_w": [b.weight.detach().cpu().clone().requires_grad_() for b in getattr(m, "bns", [])],
+            "bn_b": [b.bias.detach().cpu().clone().requires_grad_() for b in getattr(m, "bns", [])]}
+
+
+def _params_of_sage(model):
+    m = model.model
+    return {"lin_l_w": [c.lin_l.weight.detach().cpu().clone().requires_grad_() for c in m.convs],
+            "lin_l_b": [c.lin_l.bias.detach().cpu().clone().requires_grad_() for c in m.convs],
+            "lin_r_w": [c.lin_r.weight.detach().cpu().clone().requires_grad_() for c in m.convs],
+            "bn_w": [b.weight.detach().cpu().clone().requires_grad_() for b in getattr(m, "bns", [])],
+            "bn_b": [b.bias.detach().cpu().clone().requires_grad_() for b in getattr(m, "bns", [])]}
+
+
+def _flat(params):
+    return [p for v in params.values() for p in v if p is not None]
+
+
+def test_gcn_training_loss_tracks_oracle_for_20_steps(backend):
+    """BASELINE config 1: 2-layer GCN, ER graph N=4096, avg degree 10,
+    symmetrised with self loops, sym-normalised; features 128, hidden 128, 16
+    classes, INT2, kept_frac 1.  20 SGD steps; the loss stays within 1e-3 of
+    the oracle model's at every step."""
+    n, feat, hidden, classes, steps = 4096, 128, 128, 16, 20
+    A = er_graph(n, 10, 0)
+    adj = gcn_norm(SparseTensor.from_scipy(A).set_value(None), add_self_loops=True)
+    rowptr, col, value = adj.csr()
+    graph = om.Graph(rowptr.numpy(), col.numpy(), value.numpy())
+    adj = adj.to(backend).fill_cache_()
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(n, feat, generator=g)
+    labels = torch.randint(0, classes, (n,), generator=g)
+    torch.manual_seed(7)
+    model = exact.QModule(GCN(feat, hidden, classes, 2, dropout=0.5, batch_norm=True)).to(backend).train()
+    params = _params_of_gcn(model)
+    bn_state = [(b.running_mean.detach().cpu().clone(), b.running_var.detach().cpu().clone()) for b in model.model.bns]
+    other = wire_noise(21)
+    c = om.Ctx(2, 1.0, other.noise, None)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    opt_o = torch.optim.SGD(_flat(params), lr=0.05)
+    xd, yd = x.to(backend), labels.to(backend)
+    worst = 0.0
+    for step in range(steps):
+        opt.zero_grad()
+        loss = F.cross_entropy(model(xd, adj), yd)
+        loss.backward()
+        opt.step()
+        opt_o.zero_grad()
+        loss_o = F.cross_entropy(om.gcn_forward(c, params, graph, x, 0.5, True, bn_state), labels)
+        loss_o.backward()
+        opt_o.step()
+        worst = max(worst, abs(loss.item() - loss_o.item()))
+        assert abs(loss.item() - loss_o.item()) < 1e-3, (step, loss.item(), loss_o.item())
+    assert np.isfinite(loss.item())
+    print(f"max |loss - oracle loss| over {steps} steps: {worst:.2e}")
+
+
+@pytest.mark.parametrize("kept_frac,bits", [(0.125, 2), (0.25, 1)])
+def test_sage_training_loss_tracks_oracle(backend, kept_frac, bits):
+    """GraphSAGE (mean aggregation, no edge values) with random projection:
+    the shape of BASELINE configs 4 / 5 at a size the oracle runs in seconds."""
+    config.kept_frac, config.activation_compression_bits = kept_frac, [bits]
+    n, feat, hidden, classes, steps = 1500, 100, 64, 7, 8
+    A = er_graph(n, 12, 3)
+    adj = SparseTensor.from_scipy(A).set_value(None)
+    rowptr, col, _ = adj.csr()
+    graph = om.Graph(rowptr.numpy(), col.numpy(), None)
+    adj = adj.to(backend).fill_cache_()
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(n, feat, generator=g)
+    labels = torch.randint(0, classes, (n,), generator=g)
+    torch.manual_seed(8)
+    model = exact.QModule(SAGE(feat, hidden, classes, 3, dropout=0.5, batch_norm=False)).to(backend).train()
+    params = _params_of_sage(model)
+    other = wire_noise(33)
+    c = om.Ctx(bits, kept_frac, other.noise, other.rademacher)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    opt_o = torch.optim.SGD(_flat(params), lr=0.05)
+    xd, yd = x.to(backend), labels.to(backend)
+    for step in range(steps):
+        opt.zero_grad()
+        loss = F.cross_entropy(model(xd, adj), yd)
+        loss.backward()
+        opt.step()
+        opt_o.zero_grad()
+        loss_o = F.cross_entropy(om.sage_forward(c, params, graph, x, 0.5), labels)
+        loss_o.backward()
+        opt_o.step()
+        assert abs(loss.item() - loss_o.item()) < 1e-3, (step, loss.item(), loss_o.item())
+
+
+def test_qmodule_conversion_and_state_dict(backend):
+    net = GCN(16, 32, 4, 3, dropout=0.3, batch_norm=True)
+    ref_keys = list(net.state_dict().keys())
+    q = exact.QModule(net)
+    kinds = [type(m).__name__ for m in q.model.modules()]
+    assert kinds.count("QGCNConv") == 3 and kinds.count("QBatchNorm1d") == 2
+    assert "QReLU" in kinds and "QDropout" in kinds and "GCNConv" not in kinds
+    assert [k for k in q.state_dict().keys()] == ref_keys       # the "model." prefix is stripped
+    q.load_state_dict(q.state_dict())
+    s = exact.QModule(SAGE(16, 32, 4, 2))
+    names = [type(m).__name__ for m in s.model.modules()]
+    assert names.count("QSAGEConv") == 2 and names.count("QLinear") == 4
+    config.dropout2 = True
+    assert "QDropout2" in [type(m).__name__ for m in exact.QModule(GCN(4, 4, 2, 2, dropout=0.1)).model.modules()]
+    # eval mode bypasses every compressed path and equals the stock layers' arithmetic
+    q = q.to(backend).eval()
+    A = er_graph(50, 4, 1)
+    adj = gcn_norm(SparseTensor.from_scipy(A).set_value(None)).to(backend)
+    out = q(torch.randn(50, 16, device=backend), adj)
+    assert out.shape == (50, 4) and torch.isfinite(out).all()
