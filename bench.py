@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Benchmark of the activation pack/unpack hot path on one MI355X.
+"""Benchmark of EXACT's activation pack/unpack hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
@@ -9,7 +9,7 @@ every bit width {1,2,4,8}: per-row min/range + stochastic-rounding quantise +
 bit-pack (internal Philox noise), then unpack + dequantise with the bf16
 scale/min -- eight kernel launches through the C ABI of libexact_hip.so on
 preallocated buffers.  `value` is the algorithmic bytes of a step divided by
-its time.  Prints ONE JSON line; everything else goes to stderr.
+its time.  Prints ONE JSON line on stdout; progress goes to stderr.
 """
 import argparse
 import json
@@ -38,51 +38,73 @@ def packed_bytes(N, G, b):
 
 
 def algo_bytes_pack(N, G, b, supplied_noise=False):
-    # read x (+ noise), write packed + bf16 scale/min
+    """read x (+ noise), write the packed stream + bf16 scale and min"""
     return 4 * N * G * (2 if supplied_noise else 1) + packed_bytes(N, G, b) + 4 * N
 
 
 def algo_bytes_unpack(N, G, b):
+    """read the packed stream + bf16 scale and min, write fp32 [N, G]"""
     return packed_bytes(N, G, b) + 4 * N + 4 * N * G
 
 
-def main():
+def cpu_baseline(x_host, step_bytes, seed, min_seconds=10.0, max_passes=20):
+    """The C restatement of the reference algorithm (oracle/exact_oracle.c,
+    OpenMP) on the same workload, timed on this machine's host cores."""
+    import c_oracle
+    N, G = x_host.shape
+    threads = c_oracle.num_threads()
+    c_oracle.pack_unpack_roundtrip(x_host[:4096], 2, None, seed, 0)  # warm up the thread pool
+    t0 = time.perf_counter()
+    passes = 0
+    while True:
+        for b in BITS:
+            c_oracle.pack_unpack_roundtrip(x_host, b, None, seed, passes)
+        passes += 1
+        if time.perf_counter() - t0 > min_seconds or passes >= max_passes:
+            break
+    cpu_s = (time.perf_counter() - t0) / passes
+    return {"value": step_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{passes} full steps of the same workload ([{N},{G}] fp32, bits 1/2/4/8, pack+unpack, Philox "
+                      f"noise) with oracle/exact_oracle.c (OpenMP, {threads} threads), including the reference's "
+                      f"separate min and max passes (ops.py:61-66); bytes counted as for the GPU",
+            "seconds_per_step": cpu_s, "host_cpus": os.cpu_count()}
+
+
+def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--rows", type=int, default=N_ROWS, help=argparse.SUPPRESS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    args = ap.parse_args()
+    ap.add_argument("--extras-scale", type=float, default=1.0, help=argparse.SUPPRESS)
+    args = ap.parse_args(argv)
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists, "
-                 "see DESIGN.md for how the path would shard)")
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (the path has no multi-GPU code; "
+                 "DESIGN.md says how it would shard)")
 
     import torch
-    from exact_amd import _lib
+    from exact_amd import _lib, benchmarks
+    from exact_amd.cpp_extension import _checks
 
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
     L = _lib.lib()  # raises if the HIP library is missing: there is no fallback
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    stream = torch.cuda.current_stream()
-    sp = stream.cuda_stream
-
-    N, G = N_ROWS, N_COLS
+    dev = benchmarks.bench_device()
+    N, G = args.rows, N_COLS
     gen = torch.Generator(device=dev).manual_seed(1234)
     x = torch.randn((N, G), generator=gen, device=dev, dtype=torch.float32)
     out = torch.empty_like(x)
+    sp = _checks.stream_ptr(x)
     packed = {b: torch.empty(int(L.exact_packed_nbytes(N, G, b)), dtype=torch.int8, device=dev) for b in BITS}
     sbf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     mbf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     seed = 0x5EED
     calls = [0]
 
-    def pack(b, noise=None):
+    def pack(b):
         calls[0] += 1
-        rc = L.exact_minmax_pack_f32(x.data_ptr(), noise.data_ptr() if noise is not None else None, seed,
-                                     calls[0], N, G, b, packed[b].data_ptr(), None, None, sbf.data_ptr(),
-                                     mbf.data_ptr(), sp)
+        rc = L.exact_minmax_pack_f32(x.data_ptr(), None, seed, calls[0], N, G, b, packed[b].data_ptr(), None, None,
+                                     sbf.data_ptr(), mbf.data_ptr(), sp)
         assert rc == 0, rc
 
     def unpack(b):
@@ -97,44 +119,36 @@ def main():
 
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
+    benchmarks._sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
-    torch.cuda.synchronize()
+    benchmarks._sync()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     step_bytes = sum(algo_bytes_pack(N, G, b) + algo_bytes_unpack(N, G, b) for b in BITS)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    log(f"pack+unpack, bits 1/2/4/8: {ms_per_step:.3f} ms/step, {value:.1f} GB/s = {100 * value / HBM_PEAK_GBS:.1f}% of HBM peak")
 
-    # ---- per-kernel durations, HIP events on the launch stream --------------
-    def time_kernel(fn, reps=50):
-        for _ in range(5):
-            fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(reps):
-            fn()
-        e1.record(stream)
-        e1.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e-3  # seconds per launch
-
+    # ---- per-kernel durations, HIP events on the launch stream ----------------
     kernels = []
     for b in BITS:
-        tp = time_kernel(lambda: pack(b))
-        tu = time_kernel(lambda: unpack(b))
-        kernels.append({"kernel": f"pack_kernel<bits={b}> (min/max+quantise+pack, Philox noise)", "us": tp * 1e6,
+        tp = benchmarks.event_time(lambda: pack(b), reps=50, warm=5)
+        tu = benchmarks.event_time(lambda: unpack(b), reps=50, warm=5)
+        kernels.append({"kernel": f"pack_kernel<bits={b}>", "does": "row min/max + scale + stochastic quantise + "
+                        "bit-pack + bf16 scale/min, Philox noise", "us": tp * 1e6,
                         "algo_bytes": algo_bytes_pack(N, G, b), "GB/s": algo_bytes_pack(N, G, b) / tp / 1e9})
-        kernels.append({"kernel": f"unpack_kernel<bits={b}> (unpack+dequantise, bf16 scale/min)", "us": tu * 1e6,
-                        "algo_bytes": algo_bytes_unpack(N, G, b), "GB/s": algo_bytes_unpack(N, G, b) / tu / 1e9})
+        kernels.append({"kernel": f"unpack_kernel<bits={b}>", "does": "unpack + dequantise with bf16 scale/min",
+                        "us": tu * 1e6, "algo_bytes": algo_bytes_unpack(N, G, b),
+                        "GB/s": algo_bytes_unpack(N, G, b) / tu / 1e9})
     for k in kernels:
         k["frac_hbm_peak"] = k["GB/s"] / HBM_PEAK_GBS
-        log(f"  {k['kernel']:<70s} {k['us']:8.1f} us  {k['GB/s']:8.1f} GB/s  {100 * k['frac_hbm_peak']:5.1f}% of HBM peak")
+        log(f"  {k['kernel']:<24s} {k['us']:8.1f} us  {k['GB/s']:8.1f} GB/s  {100 * k['frac_hbm_peak']:5.1f}% of HBM peak")
     dom = max(kernels, key=lambda k: k["us"])
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(dom["kernel"].split(" ")[0])
+        traffic = json.load(open(tpath)).get(dom["kernel"])
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": dom["GB/s"] / HBM_PEAK_GBS, "traffic": traffic,
                 "avg_launch_us": dom["us"], "algo_bytes_per_launch": dom["algo_bytes"]}
@@ -142,48 +156,34 @@ def main():
     extras = {}
     if not args.no_extras:
         try:
-            from exact_amd import bench_extras
-            extras = bench_extras.run(L, x, log)
-        except Exception as e:  # extras never invalidate the headline line
+            extras = benchmarks.run(x, log, scale=args.extras_scale)
+        except Exception as e:  # noqa: BLE001 -- extras never invalidate the headline line
             log(f"extras failed: {type(e).__name__}: {e}")
             extras = {"error": f"{type(e).__name__}: {e}"}
 
-    # ---- CPU baseline: the C restatement of the reference algorithm ----------
     cpu = None
     if not args.no_cpu_baseline:
-        import numpy as np
-        import c_oracle
-        xs = x.cpu().numpy()
-        threads = c_oracle.num_threads()
-        c_oracle.pack_unpack_roundtrip(xs[:4096], 2, None, seed, 0)  # warm
-        t0 = time.perf_counter()
-        passes = 0
-        while True:
-            for b in BITS:
-                c_oracle.pack_unpack_roundtrip(xs, b, None, seed, passes)
-            passes += 1
-            if time.perf_counter() - t0 > 10.0 or passes >= 20:
-                break
-        cpu_s = (time.perf_counter() - t0) / passes
-        cpu = {"value": step_bytes / cpu_s / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": f"{passes} full steps of the same workload ([{N},{G}] fp32, bits 1/2/4/8, pack+unpack, "
-                         f"Philox noise) with oracle/exact_oracle.c (OpenMP, {threads} threads; the reference's "
-                         f"extra min and max passes are included, as in its ops.py:61-66)",
-               "seconds_per_step": cpu_s, "host_cpus": os.cpu_count()}
-        log(f"  cpu baseline: {cpu['value']:.2f} GB/s on {threads} threads ({cpu_s:.2f} s/step)")
+        try:
+            cpu = cpu_baseline(x.cpu().numpy(), step_bytes, seed)
+            log(f"  cpu baseline: {cpu['value']:.2f} GB/s on {cpu['cores']} threads ({cpu['seconds_per_step']:.2f} s/step)")
+        except Exception as e:  # noqa: BLE001
+            log(f"cpu baseline failed: {type(e).__name__}: {e}")
 
     result = {
         "metric": "pack+unpack GB/s (% HBM peak); INT2 GCN/SAGE full-batch epochs/s",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32->u1/u2/u4/u8 (fp32 arithmetic)", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config 2: fp32 activation [169343 x 256] ~N(0,1); per-row min/range + stochastic "
-                               "quantise + pack, then unpack + dequantise, at bits {1,2,4,8}; internal Philox noise",
+                               "quantise + bit-pack, then unpack + dequantise, at bits {1,2,4,8}; internal Philox "
+                               "noise; inputs resident in HBM",
                    "rows": N, "cols": G, "bits": list(BITS), "algo_bytes_per_step": step_bytes},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
+        "epochs_per_s": {k: v.get("epochs_per_s") for k, v in extras.items() if isinstance(v, dict) and k.startswith("cfg")},
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "extras": extras,
     }
-    print(json.dumps(result))
+    print(json.dumps(result), flush=True)
+    return result
 
 
 if __name__ == "__main__":

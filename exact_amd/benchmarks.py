@@ -1,0 +1,271 @@
+"""Measurements beyond the headline pack+unpack number: the other kernels of
+the path at the benchmark shapes, and full-batch training epochs/s of the
+INT2 / INT1 GCN and GraphSAGE configurations on synthetic power-law graphs
+(the loop of mem_speed_bench/arxiv/train_full_batch.py:256-266 in the
+reference: zero_grad, forward on all nodes, nll_loss on the training nodes,
+backward, optimizer step).  bench.py calls run(); every number is measured
+with HIP events on the stream the kernels are launched on.
+"""
+from __future__ import annotations
+
+import time
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from .conf import QuantizationConfig, config
+from .cpp_extension import quantization as extq
+from .cpp_extension import spmm as ext_spmm
+from .models import GCN, SAGE
+from .module import QModule
+from .sparse import SparseTensor, gcn_norm
+
+HBM_PEAK_GBS = 8000.0
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+def event_time(fn, reps=20, warm=3):
+    """Average seconds per call of fn(), HIP events on the current stream."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / reps * 1e-3
+
+
+def bench_device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("the benchmarks need a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    return dev
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+def _reset_peak(device):
+    torch.cuda.reset_peak_memory_stats(device)
+
+
+def _peak_gb(device):
+    return torch.cuda.max_memory_allocated(device) / 1e9
+
+
+def _trim():
+    torch.cuda.empty_cache()
+
+
+def powerlaw_graph(n, target_directed_edges, seed, device, alpha=2.1, max_degree=None):
+    """Synthetic power-law graph: out-degree ~ Pareto tail with exponent alpha
+    (the continuous stand-in for Zipf), rescaled to about
+    `target_directed_edges` raw edges, uniformly random targets, then
+    symmetrised and de-duplicated.  Returns an unvalued SparseTensor (CSR)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    u = torch.rand(n, generator=g, device=device).clamp_(min=1e-9)
+    raw = u.pow(-1.0 / (alpha - 1.0))
+    cap = float(max_degree if max_degree is not None else max(64, n // 16))
+    raw.clamp_(max=cap)
+    deg = (raw * (target_directed_edges / raw.sum())).round().clamp_(min=1, max=cap).long()
+    src = torch.repeat_interleave(torch.arange(n, device=device), deg)
+    dst = torch.randint(0, n, (src.numel(),), generator=g, device=device)
+    keep = src != dst
+    src, dst = src[keep], dst[keep]
+    key = torch.cat([src * n + dst, dst * n + src]).unique()        # symmetrise, drop duplicates (sorted)
+    row, col = torch.div(key, n, rounding_mode="floor"), key % n
+    rowptr = torch.zeros(n + 1, dtype=torch.long, device=device)
+    torch.cumsum(torch.bincount(row, minlength=n), 0, out=rowptr[1:])
+    adj = SparseTensor(rowptr, col, None, (n, n))
+    adj.storage._row = row
+    return adj
+
+
+def spmm_bytes(M, n_cols, nnz, K, idx_bytes, valued):
+    """Compulsory traffic: index arrays + values + X once + output once."""
+    return (M + 1) * idx_bytes + nnz * (idx_bytes + (4 if valued else 0)) + 4 * n_cols * K + 4 * M * K
+
+
+def kernel_extras(x, log):
+    """Masks, projection GEMMs and supplied-noise pack at the config-2 shape."""
+    out = {}
+    N, G = x.shape
+    n = N * G
+    saved = dict(config.__dict__)
+    try:
+        config.__dict__.update(QuantizationConfig().__dict__)
+        # --- 1-bit masks ---------------------------------------------------
+        mask_bytes = 8 * n + n // 8
+        xr = x.clone().requires_grad_()
+        y = extq.act_quantized_relu(xr)
+        gy = torch.ones_like(y)
+        t = event_time(lambda: extq.act_quantized_relu(x))
+        out["relu_fwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
+        t = event_time(lambda: torch.autograd.grad(y, xr, gy, retain_graph=True))
+        out["relu_bwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
+        t = event_time(lambda: extq.act_quantized_dropout(x, 0.5, True))
+        out["dropout_fwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
+        yd = extq.act_quantized_dropout(xr, 0.5, True)
+        t = event_time(lambda: torch.autograd.grad(yd, xr, gy, retain_graph=True))
+        out["dropout_bwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
+        del y, yd, gy, xr
+        # --- random projection 256 -> 32 (kept_frac 0.125), Gaussian N(0, 1/k) --
+        k = int(0.125 * G + 0.999)
+        R = torch.randn(G, k, device=x.device) / k ** 0.5
+        config.rp_matrix_source = lambda D_, k_, device: R
+        rp_bytes = 4 * N * G + 4 * G * k + 4 * N * k
+        flops = 2.0 * N * G * k
+        xr_small, _ = ops.input2rp(x, k)
+        t = event_time(lambda: ops.input2rp(x, k))
+        out["rp_fwd"] = {"us": t * 1e6, "GB/s": rp_bytes / t / 1e9, "TFLOP/s": flops / t / 1e12,
+                         "mfma_frac_of_fp32_peak": flops / t / 1e12 / FP32_MFMA_PEAK_TFLOPS, "algo_bytes": rp_bytes}
+        t = event_time(lambda: ops.rp2input(xr_small, x.shape, R))
+        out["rp_bwd"] = {"us": t * 1e6, "GB/s": rp_bytes / t / 1e9, "TFLOP/s": flops / t / 1e12,
+                         "mfma_frac_of_fp32_peak": flops / t / 1e12 / FP32_MFMA_PEAK_TFLOPS, "algo_bytes": rp_bytes}
+        # compress = project + quantise + pack of the reduced tensor, and back
+        config.kept_frac, config.rp_matrix_source = 0.125, (lambda D_, k_, device: R)
+        q = ops.quantize_activation(xr_small, None)
+        t = event_time(lambda: ops.quantize_activation(ops.input2rp(x, k)[0], None))
+        out["rp_compress_int2"] = {"us": t * 1e6}
+        t = event_time(lambda: ops.rp2input(ops.dequantize_activation(q, xr_small.shape), x.shape, R))
+        out["rp_decompress_int2"] = {"us": t * 1e6}
+        for name, v in out.items():
+            if "GB/s" in v:
+                v["frac_hbm_peak"] = v["GB/s"] / HBM_PEAK_GBS
+            log(f"  {name:<22s} {v['us']:9.1f} us" + (f"  {v['GB/s']:8.1f} GB/s" if "GB/s" in v else ""))
+    finally:
+        config.__dict__.clear()
+        config.__dict__.update(saved)
+    return out
+
+
+def spmm_extras(adj, K, log, valued_norm=True):
+    """Forward and transpose-backward SpMM on one graph at width K."""
+    dev = adj.device()
+    rowptr, col, value = adj.csr()
+    M = adj.sparse_size(0)
+    nnz = col.numel()
+    X = torch.randn(M, K, device=dev)
+    st = adj.storage
+    reduce = "sum" if value is not None else "mean"
+    t_fw = event_time(lambda: ext_spmm.spmm_csr(rowptr, col, value, X, reduce), reps=10)
+    if reduce == "sum":
+        bw = lambda: ext_spmm.spmm_sum_bw(st.row(), rowptr, col, value, st.colptr(), st.csr2csc(), None, X,  # noqa: E731
+                                          value is not None, False, True)
+    else:
+        bw = lambda: ext_spmm.spmm_mean_bw(st.row(), rowptr, col, value, st.rowcount(), st.colptr(), st.csr2csc(),  # noqa: E731
+                                           None, X, value is not None, False, True)
+    t_bw = event_time(bw, reps=10)
+    b = spmm_bytes(M, M, nnz, K, rowptr.element_size(), value is not None)
+    b_bw = spmm_bytes(M, M, nnz, K, rowptr.element_size(), True)
+    res = {"rows": M, "nnz": nnz, "K": K, "reduce": reduce, "index_bytes": rowptr.element_size(),
+           "fwd_us": t_fw * 1e6, "bwd_us": t_bw * 1e6, "compulsory_bytes": b,
+           "fwd_GB/s_compulsory": b / t_fw / 1e9, "bwd_GB/s_compulsory": b_bw / t_bw / 1e9,
+           "fwd_frac_hbm_peak": b / t_fw / 1e9 / HBM_PEAK_GBS,
+           "gather_bytes_no_reuse": 4 * nnz * K, "fwd_GB/s_gather": 4 * nnz * K / t_fw / 1e9,
+           "fwd_GFLOP/s": 2.0 * nnz * K / t_fw / 1e9}
+    log(f"  spmm {reduce} M={M} nnz={nnz} K={K}: fwd {t_fw * 1e6:.0f} us ({res['fwd_GB/s_compulsory']:.0f} GB/s compulsory, "
+        f"{res['fwd_GB/s_gather']:.0f} GB/s gathered), bwd {t_bw * 1e6:.0f} us")
+    return res
+
+
+def train_epochs(model, x, adj, labels, train_idx, epochs, warmup, lr=0.01):
+    """The reference's --test_speed loop; returns (epochs/s, last loss)."""
+    opt = torch.optim.Adam(model.parameters(), lr=lr)
+    model.train()
+
+    def one():
+        opt.zero_grad()
+        out = F.log_softmax(model(x, adj)[train_idx], dim=-1)
+        loss = F.nll_loss(out, labels[train_idx])
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(warmup):
+        one()
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(epochs):
+        loss = one()
+    _sync()
+    dt = time.perf_counter() - t0
+    return epochs / dt, float(loss.detach())
+
+
+EPOCH_CONFIGS = {
+    # name: (model, N, raw directed edges, features, hidden, classes, layers, bits, kept_frac, batch_norm, dropout)
+    "cfg3_gcn_int2": ("gcn", 169343, 1_160_000, 128, 256, 40, 3, 2, 1.0, True, 0.5),
+    "cfg4_sage_int2_rp0.125": ("sage", 232965, 11_600_000, 602, 256, 41, 2, 2, 0.125, False, 0.5),
+    "cfg5_sage_int1_rp0.25": ("sage", 2449029, 61_900_000, 100, 256, 47, 3, 1, 0.25, False, 0.5),
+}
+
+
+def epoch_benchmark(name, device, log, epochs=10, warmup=3, int32_index=True, scale=1.0):
+    kind, n, edges, feat, hidden, classes, layers, bits, kept_frac, bn, dropout = EPOCH_CONFIGS[name]
+    n, edges = int(n * scale), int(edges * scale)
+    saved = dict(config.__dict__)
+    try:
+        config.__dict__.update(QuantizationConfig().__dict__)
+        config.activation_compression_bits, config.kept_frac = [bits], kept_frac
+        t0 = time.perf_counter()
+        adj = powerlaw_graph(n, edges, seed=1, device=device)
+        if kind == "gcn":
+            adj = gcn_norm(adj, add_self_loops=True)
+        if int32_index:
+            adj.to_int32_()
+        adj.fill_cache_()
+        nnz = adj.nnz()
+        g = torch.Generator(device=device).manual_seed(2)
+        x = torch.randn(n, feat, generator=g, device=device)
+        labels = torch.randint(0, classes, (n,), generator=g, device=device)
+        train_idx = torch.randperm(n, generator=g, device=device)[: n // 2]
+        torch.manual_seed(3)
+        if kind == "gcn":
+            net = GCN(feat, hidden, classes, layers, dropout=dropout, batch_norm=bn)
+        else:
+            net = SAGE(feat, hidden, classes, layers, dropout=dropout, batch_norm=bn)
+        model = QModule(net).to(device)
+        _sync()
+        setup_s = time.perf_counter() - t0
+        _reset_peak(device)
+        eps, loss = train_epochs(model, x, adj, labels, train_idx, epochs, warmup)
+        res = {"epochs_per_s": eps, "ms_per_epoch": 1e3 / eps, "nodes": n, "nnz": nnz, "features": feat,
+               "hidden": hidden, "classes": classes, "layers": layers, "bits": bits, "kept_frac": kept_frac,
+               "index_dtype": "int32" if int32_index else "int64", "epochs_timed": epochs, "last_loss": loss,
+               "setup_s": setup_s, "peak_mem_GB": _peak_gb(device)}
+        log(f"  {name}: {eps:.2f} epochs/s ({1e3 / eps:.1f} ms/epoch), N={n}, nnz={nnz}, peak {res['peak_mem_GB']:.1f} GB")
+        res["spmm"] = spmm_extras(adj, hidden if kind == "gcn" else feat, log)
+        return res
+    finally:
+        config.__dict__.clear()
+        config.__dict__.update(saved)
+        ext_spmm.clear_csc_cache()
+
+
+def run(x, log, budget_s=240.0, epoch_configs=("cfg3_gcn_int2", "cfg4_sage_int2_rp0.125", "cfg5_sage_int1_rp0.25"),
+        scale=1.0, epochs=10, warmup=3):
+    """Everything beyond the headline number; each part is independent and a
+    failure or an exhausted time budget in one only drops that part."""
+    t_start = time.perf_counter()
+    out = {}
+    try:
+        out["kernels"] = kernel_extras(x, log)
+    except Exception as e:  # noqa: BLE001
+        out["kernels"] = {"error": f"{type(e).__name__}: {e}"}
+    _trim()
+    for name in epoch_configs:
+        if time.perf_counter() - t_start > budget_s:
+            out[name] = {"skipped": "time budget of the default run exhausted"}
+            continue
+        try:
+            out[name] = epoch_benchmark(name, x.device, log, epochs=epochs, warmup=warmup, scale=scale)
+        except Exception as e:  # noqa: BLE001
+            out[name] = {"error": f"{type(e).__name__}: {e}"}
+        _trim()
+    return out
