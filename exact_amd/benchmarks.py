@@ -269,3 +269,69 @@ def run(x, log, budget_s=240.0, epoch_configs=("cfg3_gcn_int2", "cfg4_sage_int2_
             out[name] = {"error": f"{type(e).__name__}: {e}"}
         _trim()
     return out
+
+
+def _profile_target(argv=None):
+    """One kernel in a loop, as the target of `rocprofv3 --kernel-trace --stats` /
+    `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
+
+        python -m exact_amd.benchmarks pack --bits 2 --reps 100
+        python -m exact_amd.benchmarks {unpack,relu,dropout,rp_fwd,rp_bwd,spmm,copy} ...
+
+    `copy` is a plain device-to-device copy of the same [rows, cols] fp32 tensor
+    (4*rows*cols bytes read, as many written) for calibrating the byte counters."""
+    import argparse
+
+    from . import _lib
+    from .cpp_extension import _checks
+    ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
+    ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "rp_fwd", "rp_bwd", "spmm", "copy"])
+    ap.add_argument("--bits", type=int, default=2)
+    ap.add_argument("--rows", type=int, default=169343)
+    ap.add_argument("--cols", type=int, default=256)
+    ap.add_argument("--reps", type=int, default=100)
+    ap.add_argument("--supplied-noise", action="store_true")
+    args = ap.parse_args(argv)
+    dev = bench_device()
+    L = _lib.lib()
+    N, G, b = args.rows, args.cols, args.bits
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    x = torch.randn((N, G), generator=gen, device=dev)
+    sp = _checks.stream_ptr(x)
+    out = torch.empty_like(x)
+    packed = torch.empty(int(L.exact_packed_nbytes(N, G, b)), dtype=torch.int8, device=dev)
+    sbf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    mbf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    noise = torch.rand((N, G), generator=gen, device=dev) if args.supplied_noise else None
+    mask = torch.empty((N * G + 31) // 32, dtype=torch.int32, device=dev)
+    L.exact_minmax_pack_f32(x.data_ptr(), None, 1, 1, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),
+                            mbf.data_ptr(), sp)
+    k = int(0.125 * G + 0.999)
+    R = torch.randn(G, k, generator=gen, device=dev) / k ** 0.5
+    xr = torch.empty((N, k), device=dev)
+    if args.kernel == "spmm":
+        adj = gcn_norm(powerlaw_graph(N, int(N * 6.85), seed=1, device=dev)).to_int32_()
+        rowptr, col, value = adj.csr()
+    fns = {
+        "pack": lambda i: L.exact_minmax_pack_f32(x.data_ptr(), noise.data_ptr() if noise is not None else None, 1,
+                                                  i, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),
+                                                  mbf.data_ptr(), sp),
+        "unpack": lambda i: L.exact_unpack_bf16param_f32(packed.data_ptr(), b, sbf.data_ptr(), mbf.data_ptr(), N, G,
+                                                         out.data_ptr(), sp),
+        "relu": lambda i: L.exact_relu_fwd_f32(x.data_ptr(), N * G, out.data_ptr(), mask.data_ptr(), sp),
+        "dropout": lambda i: L.exact_dropout_fwd_f32(x.data_ptr(), None, 1, i, 0.5, N * G, out.data_ptr(),
+                                                     mask.data_ptr(), sp),
+        "rp_fwd": lambda i: L.exact_rp_fwd_f32(x.data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp),
+        "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, out.data_ptr(), sp),
+        "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, x, "sum"),
+        "copy": lambda i: out.copy_(x),
+    }
+    fn = fns[args.kernel]
+    for i in range(args.reps):
+        fn(i + 2)
+    _sync()
+    print(f"{args.kernel}: {args.reps} launches on [{N}, {G}] done")
+
+
+if __name__ == "__main__":
+    _profile_target()

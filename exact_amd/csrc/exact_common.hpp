@@ -89,8 +89,29 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
 // ---- cross-lane ------------------------------------------------------------
 // Butterfly min / max over aligned groups of `span` lanes (span a power of two
 // <= 64).  Every lane of the group ends with the group's result.
+// The first three steps stay inside the VALU as DPP moves: quad_perm [1,0,3,2]
+// and [2,3,0,1] fold a quad, after which all four lanes of a quad agree, so the
+// half-row mirror (lane i <-> 7 - i) delivers "the other quad" to every lane.
+// Wider steps go through the LDS crossbar (__shfl_xor).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
 __device__ __forceinline__ void group_minmax(float& mn, float& mx, int span) {
-  for (int m = 1; m < span; m <<= 1) {
+  if (span >= 2) {
+    mn = fminf(mn, dpp_move<0xB1>(mn));
+    mx = fmaxf(mx, dpp_move<0xB1>(mx));
+  }
+  if (span >= 4) {
+    mn = fminf(mn, dpp_move<0x4E>(mn));
+    mx = fmaxf(mx, dpp_move<0x4E>(mx));
+  }
+  if (span >= 8) {
+    mn = fminf(mn, dpp_move<0x141>(mn));
+    mx = fmaxf(mx, dpp_move<0x141>(mx));
+  }
+  for (int m = 8; m < span; m <<= 1) {
     mn = fminf(mn, __shfl_xor(mn, m));
     mx = fmaxf(mx, __shfl_xor(mx, m));
   }

@@ -79,7 +79,7 @@ template <int BITS, int OPT, int VEC, bool FULL, bool NOISE_IN, bool FUSED>
 __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   constexpr int WPT = 8 / BITS;
   constexpr float B = static_cast<float>((1 << BITS) - 1);
-  __shared__ uint2 stage[OPT * kBlock];
+  __shared__ uint2 stage[WPT > 1 ? OPT * kBlock : 1];
 
   const int t = threadIdx.x;
   const int lpr = 1 << a.lpr_log2;
@@ -138,6 +138,7 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
     }
   }
 
+  uint2 codes[OPT];
 #pragma unroll
   for (int k = 0; k < OPT; ++k) {
     const int j = oct_base + lane_in_row + k * lpr;
@@ -166,10 +167,11 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       const uint32_t qi = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
       q[i] = ((FULL ? row_ok : (i < nv[k])) ? qi : 0u) & 0xFFu;
     }
-    stage[k * kBlock + t] = make_uint2(q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24),
-                                       q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24));
+    codes[k] = make_uint2(q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24),
+                          q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24));
+    if constexpr (WPT > 1) stage[k * kBlock + t] = codes[k];
   }
-  __syncthreads();
+  if constexpr (WPT > 1) __syncthreads();  // 8-bit codes: one row per byte, nothing to combine
 
   // The lane holding the first row of a row-group packs the whole group.
   if ((row_local & (WPT - 1)) == 0 && row_ok) {
@@ -177,9 +179,9 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
     for (int k = 0; k < OPT; ++k) {
       const int j = oct_base + lane_in_row + k * lpr;
       if (j >= a.opr) continue;
-      uint32_t w0 = 0, w1 = 0;
+      uint32_t w0 = codes[k].x, w1 = codes[k].y;
 #pragma unroll
-      for (int i = 0; i < WPT; ++i) {
+      for (int i = 1; i < WPT; ++i) {
         // uint8 accumulator of the reference: bits shifted past bit 7 vanish
         constexpr uint32_t kByte = 0x01010101u;
         const uint32_t keep = (0xFFu >> (i * BITS)) * kByte;

@@ -180,6 +180,7 @@ static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
 }
 
 int main(int argc, char** argv) {
+  std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
   std::mt19937 rng(12345);
   const int64_t shapes[][2] = {{1, 1}, {5, 3}, {37, 25}, {64, 32}, {100, 76}, {33, 40}, {129, 100}, {300, 128},

