@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE config 2): an fp32 activation [169343, 256] ~ N(0,1)
+Workload (the op-level microbenchmark configuration): an fp32 activation [169343, 256] ~ N(0,1)
 resident in HBM.  One step = quantize_activation + dequantize_activation at
 every bit width {1,2,4,8}: per-row min/range + stochastic-rounding quantise +
 bit-pack (internal Philox noise), then unpack + dequantise with the bf16
@@ -82,7 +82,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (the path has no multi-GPU code; "
-                 "DESIGN.md says how it would shard)")
+                 "row blocks aligned to 8 rows would shard it without communication)")
 
     import torch
     from exact_amd import _lib, benchmarks

@@ -136,3 +136,39 @@ def test_rp(N, D, frac, dist):
     back = e.rp_bwd(got, R)
     wb = o.rp2input(got, R)
     np.testing.assert_allclose(back, wb, rtol=1e-5, atol=1e-5 * np.abs(wb).max())
+
+
+def test_pack_unpack_random_shapes():
+    """Randomly drawn shapes (any N, any G up to a few thousand, every bit
+    width, both noise modes): the fixed list above cannot enumerate every
+    remainder of N mod 8 and G mod 8 against every lanes-per-row choice."""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        bits = int(rng.choice([1, 2, 4, 8]))
+        N = int(rng.integers(1, 70))
+        G = int(rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(300, 1100), rng.integers(1100, 2600)]))
+        x = (rng.standard_normal((N, G)) * rng.uniform(0.1, 10)).astype(F32)
+        u = rng.random((N, G), dtype=F32)
+        want = o.quantize_activation(x, bits, u)
+        packed, s32, m32, sbf, mbf = e.minmax_pack(x, bits, u)
+        assert np.array_equal(packed, want[0]), (case, bits, N, G)
+        assert np.array_equal(sbf, want[2]) and np.array_equal(mbf, want[3]), (case, bits, N, G)
+        xh = e.unpack(packed, bits, sbf, mbf, N, G, bf16=True)
+        ref = o.dequantize_activation(want[0], bits, want[2], want[3], (N, G))
+        assert np.array_equal(xh.view(np.uint32), ref.view(np.uint32)), (case, bits, N, G)
+        seed, off = int(rng.integers(0, 2 ** 63)), int(rng.integers(0, 2 ** 63))
+        got = e.minmax_pack(x, bits, None, seed, off)[0]
+        assert np.array_equal(got, o.quantize_activation(x, bits, o.philox_noise_rows(seed, off, N, G))[0]), (case, bits, N, G)
+
+
+def test_masks_random_sizes():
+    rng = np.random.default_rng(7)
+    for n in rng.integers(1, 9000, 25).tolist():
+        x = rng.standard_normal(n).astype(F32)
+        y, mask = e.relu_fwd(x)
+        wy, wm = o.relu_fwd(x)
+        assert np.array_equal(y, wy) and np.array_equal(mask, wm), n
+        seed, off = int(rng.integers(0, 2 ** 63)), int(rng.integers(0, 2 ** 63))
+        y, mask = e.dropout_fwd(x, 0.3, None, seed, off)
+        wy, wm = o.dropout_fwd(x, 0.3, o.philox_noise_flat(seed, off, n))
+        assert np.array_equal(y.view(np.uint32), wy.view(np.uint32)) and np.array_equal(mask, wm), n

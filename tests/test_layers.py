@@ -173,7 +173,7 @@ def _flat(params):
 
 
 def test_gcn_training_loss_tracks_oracle_for_20_steps(backend):
-    """BASELINE config 1: 2-layer GCN, ER graph N=4096, avg degree 10,
+    """The plumbing configuration: 2-layer GCN, ER graph N=4096, avg degree 10,
     symmetrised with self loops, sym-normalised; features 128, hidden 128, 16
     classes, INT2, kept_frac 1.  20 SGD steps; the loss stays within 1e-3 of
     the oracle model's at every step."""
@@ -214,7 +214,7 @@ def test_gcn_training_loss_tracks_oracle_for_20_steps(backend):
 @pytest.mark.parametrize("kept_frac,bits", [(0.125, 2), (0.25, 1)])
 def test_sage_training_loss_tracks_oracle(backend, kept_frac, bits):
     """GraphSAGE (mean aggregation, no edge values) with random projection:
-    the shape of BASELINE configs 4 / 5 at a size the oracle runs in seconds."""
+    the shape of the two GraphSAGE benchmark configurations at a size the oracle runs in seconds."""
     config.kept_frac, config.activation_compression_bits = kept_frac, [bits]
     n, feat, hidden, classes, steps = 1500, 100, 64, 7, 8
     A = er_graph(n, 12, 3)
