@@ -153,14 +153,6 @@ def main(argv=None):
                 "unit": "GB/s", "frac": dom["GB/s"] / HBM_PEAK_GBS, "traffic": traffic,
                 "avg_launch_us": dom["us"], "algo_bytes_per_launch": dom["algo_bytes"]}
 
-    extras = {}
-    if not args.no_extras:
-        try:
-            extras = benchmarks.run(x, log, scale=args.extras_scale)
-        except Exception as e:  # noqa: BLE001 -- extras never invalidate the headline line
-            log(f"extras failed: {type(e).__name__}: {e}")
-            extras = {"error": f"{type(e).__name__}: {e}"}
-
     cpu = None
     if not args.no_cpu_baseline:
         try:
@@ -168,6 +160,14 @@ def main(argv=None):
             log(f"  cpu baseline: {cpu['value']:.2f} GB/s on {cpu['cores']} threads ({cpu['seconds_per_step']:.2f} s/step)")
         except Exception as e:  # noqa: BLE001
             log(f"cpu baseline failed: {type(e).__name__}: {e}")
+
+    extras = {}
+    if not args.no_extras:
+        try:
+            extras = benchmarks.run(x, log, scale=args.extras_scale)
+        except Exception as e:  # noqa: BLE001 -- extras never invalidate the headline line
+            log(f"extras failed: {type(e).__name__}: {e}")
+            extras = {"error": f"{type(e).__name__}: {e}"}
 
     result = {
         "metric": "pack+unpack GB/s (% HBM peak); INT2 GCN/SAGE full-batch epochs/s",

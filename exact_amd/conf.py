@@ -1,42 +1,59 @@
-"""Global quantisation config: same singleton and field names as the
-reference's exact/exact/conf.py:1-24, read at call time by the ops."""
+"""The global quantisation config.  A mutable module-level singleton with the
+field names of the reference's QuantizationConfig (exact/exact/conf.py:3-22),
+read by the ops at call time; the trainers of the reference set these fields
+from their command lines, so the names are part of the API."""
+import copy
+
+# field -> default.  First block: the reference's fields, same defaults.
+_REFERENCE_FIELDS = {
+    "compress_activation": True,          # False: every Q-layer keeps full-precision activations
+    "activation_compression_bits": [2],   # bits per element; element 0 is the one used
+    "initial_bits": 8,
+    "stochastic": True,                   # the kernels implement stochastic rounding only
+    "use_gradient": False,
+    "simulate": False,                    # not provided here (raises when set)
+    "enable_quantized_bn": True,          # QModule swaps BatchNorm1d only when set
+    "kept_frac": 1.0,                     # < 1: random projection D -> int(kept_frac * D + 0.999)
+    "single_precision": True,             # read at layer construction: attach QScheme objects
+    "dropout2": False,                    # QModule uses QDropout2 instead of QDropout
+    "empty_cache_threshold": None,
+    "swap": False,                        # not provided here (raises when set)
+    "amp": False,
+    "debug_memory_op_forward": False,
+    "debug_memory_op_backward": False,
+    "debug_remove_bn": False,
+    "debug_remove_relu": False,
+    "debug_remove_dropout": False,
+}
+
+# Second block: additions of this implementation.
+_EXTRA_FIELDS = {
+    # Distribution of the projection matrix: "rademacher" (+-1/sqrt(k), what the
+    # reference draws, ops.py:112-114) or "gaussian" (N(0, 1/k)).
+    "rp_distribution": "rademacher",
+    # None: the kernels draw Philox noise keyed by torch's CUDA generator.  A
+    # callable (shape, device) -> fp32 uniforms in [0, 1) supplies the noise of
+    # stochastic rounding and dropout instead (parity tests feed the oracle and
+    # the kernels the same bits this way).
+    "noise_source": None,
+    # None: input2rp draws the projection matrix.  A callable (D, k, device) ->
+    # fp32 [D, k] supplies it instead.
+    "rp_matrix_source": None,
+    # The reference compresses and keeps the dense operand of every quantised
+    # SpMM although backward reads it only for edge-value gradients; set this to
+    # reproduce that memory behaviour.  Results do not depend on it.
+    "keep_unused_spmm_operand": False,
+}
 
 
 class QuantizationConfig:
     def __init__(self):
-        self.compress_activation = True
-        self.activation_compression_bits = [2]
-        self.initial_bits = 8
-        self.stochastic = True
-        self.use_gradient = False
-        self.simulate = False
-        self.enable_quantized_bn = True
-        self.kept_frac = 1.0
-        self.single_precision = True
-        self.dropout2 = False
-        # Memory management flags
-        self.empty_cache_threshold = None
-        self.swap = False
-        self.amp = False
-        # Debug flags
-        self.debug_memory_op_forward = False
-        self.debug_memory_op_backward = False
-        self.debug_remove_bn = False
-        self.debug_remove_relu = False
-        self.debug_remove_dropout = False
+        for table in (_REFERENCE_FIELDS, _EXTRA_FIELDS):
+            for name, default in table.items():
+                setattr(self, name, copy.copy(default))
 
-        # ---- additions of this implementation (not in the reference) ----
-        # Distribution of the random-projection matrix: "rademacher" is what
-        # the reference draws (ops.py:112-114); "gaussian" is N(0, 1/k).
-        self.rp_distribution = "rademacher"
-        # None: the kernels draw their own Philox noise, keyed by torch's CUDA
-        # generator.  A callable (shape, device) -> fp32 tensor of uniforms in
-        # [0, 1) supplies the noise instead (stochastic rounding and dropout);
-        # parity tests use this to feed the oracle and the kernels the same bits.
-        self.noise_source = None
-        # None: input2rp draws the projection matrix on the device.  A callable
-        # (D, k, device) -> fp32 [D, k] tensor supplies it instead.
-        self.rp_matrix_source = None
+    def __repr__(self):
+        return "QuantizationConfig(" + ", ".join(f"{k}={v!r}" for k, v in vars(self).items()) + ")"
 
 
 config = QuantizationConfig()

@@ -1,89 +1,78 @@
-"""Small helpers kept from the reference's exact/exact/utils.py: index
-down-casting (:9-28), host swap (:31-34), memory accounting (:37-65),
-allocator trimming (:68-74) and the JSON-lines recorder (:85-105)."""
+"""Small host-side helpers with the names the reference exports from
+exact/exact/utils.py: index narrowing (cast_low_bit_int / cast_adj, :9-28),
+memory accounting (get_memory_usage / compute_tensor_bytes, :37-65), allocator
+trimming (empty_cache, :68-74) and the JSON-lines experiment recorder (:85-105)."""
 import json
-from collections import OrderedDict
 
-import numpy as np
 import torch
+
+_INT32_MAX = 2 ** 31 - 1
 
 
 def cast_low_bit_int(idx_vec):
-    """int64 index vector -> int32 when every value fits (utils.py:9-19).
-    The reference also narrows to int16; the SpMM kernels here take int32 or
-    int64, so int16 is never produced."""
+    """Narrow an int64 index vector to int32 when all its values fit.  (The
+    reference also narrows to int16; the SpMM kernels here read int32 or int64.)"""
     if idx_vec is None:
-        return idx_vec
-    assert idx_vec.dtype == torch.int64
-    if idx_vec.numel() == 0 or int(idx_vec.max()) < np.iinfo(np.int32).max:
-        return idx_vec.to(torch.int32)
-    return idx_vec
+        return None
+    if idx_vec.dtype != torch.int64:
+        raise TypeError("expected an int64 index vector")
+    fits = idx_vec.numel() == 0 or int(idx_vec.max()) < _INT32_MAX
+    return idx_vec.to(torch.int32) if fits else idx_vec
 
 
 def cast_adj(data):
-    """utils.py:22-28: narrow every cached index vector of data.adj_t."""
-    st = data.adj_t.storage
-    for name in ("_col", "_row", "_rowptr", "_rowcount", "_colptr", "_csr2csc"):
-        setattr(st, name, cast_low_bit_int(getattr(st, name)))
-
-
-def swap_to_cpu(tensor):
-    tensor_cpu = torch.empty(tensor.shape, dtype=tensor.dtype, device="cpu", pin_memory=True)
-    tensor_cpu.copy_(tensor, non_blocking=True)
-    return tensor_cpu
+    """Narrow every cached index vector of data.adj_t in place."""
+    storage = data.adj_t.storage
+    for field in ("_rowptr", "_col", "_row", "_rowcount", "_colptr", "_csr2csc"):
+        setattr(storage, field, cast_low_bit_int(getattr(storage, field)))
 
 
 def get_memory_usage(gpu, print_info=False):
+    """Bytes currently allocated by torch on device `gpu`."""
     allocated = torch.cuda.memory_allocated(gpu)
-    reserved = torch.cuda.memory_reserved(gpu)
     if print_info:
-        print("allocated: %.2f MB" % (allocated / 1024 / 1024), flush=True)
-        print("reserved:  %.2f MB" % (reserved / 1024 / 1024), flush=True)
+        mib = 1 << 20
+        print(f"allocated: {allocated / mib:.2f} MB", flush=True)
+        print(f"reserved:  {torch.cuda.memory_reserved(gpu) / mib:.2f} MB", flush=True)
     return allocated
 
 
-_BYTES = {torch.int64: 8, torch.float32: 4, torch.int32: 4, torch.bfloat16: 2, torch.float16: 2,
-          torch.int16: 2, torch.int8: 1, torch.uint8: 1}
-
-
 def compute_tensor_bytes(tensors):
-    if not isinstance(tensors, (list, tuple)):
-        tensors = [tensors]
-    total = 0
-    for x in tensors:
-        if x.dtype not in _BYTES:
-            raise ValueError(x.dtype)
-        total += int(np.prod(x.size())) * _BYTES[x.dtype]
-    return total
+    """Bytes held by a tensor or a list / tuple of tensors."""
+    if isinstance(tensors, torch.Tensor):
+        tensors = (tensors,)
+    return sum(t.numel() * t.element_size() for t in tensors)
 
 
 def empty_cache(ratio):
+    """Return cached blocks to the driver when less than `ratio` of the reserved
+    memory is in use; None switches it off."""
     if ratio is None:
         return
-    allocated = torch.cuda.memory_allocated(0)
     reserved = torch.cuda.memory_reserved(0)
-    if reserved > 0 and allocated / reserved < ratio:
+    if reserved > 0 and torch.cuda.memory_allocated(0) < ratio * reserved:
         torch.cuda.empty_cache()
 
 
 class GlobalExpRecorder:
+    """Collects key/value results of one experiment and appends them to a
+    JSON-lines file."""
+
     def __init__(self):
-        self.val_dict = OrderedDict()
+        self.val_dict = {}
 
     def record(self, key, value, float_round=6):
-        if isinstance(value, (np.int32, np.int64)):
-            value = int(value)
-        if isinstance(value, (float, np.float32, np.float64)):
-            value = round(float(value), float_round)
-        self.val_dict[key] = value
+        if hasattr(value, "item"):
+            value = value.item()
+        self.val_dict[key] = round(value, float_round) if isinstance(value, float) else value
 
     def dump(self, filename):
-        with open(filename, "a") as fout:
-            fout.write(json.dumps(self.val_dict) + "\n")
-        print("Save exp results to %s" % filename)
+        with open(filename, "a") as out:
+            out.write(json.dumps(self.val_dict) + "\n")
+        print(f"Save exp results to {filename}")
 
     def clear(self):
-        pass
+        self.val_dict.clear()
 
 
 exp_recorder = GlobalExpRecorder()
