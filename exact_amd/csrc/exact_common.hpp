@@ -95,7 +95,7 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
 // Wider steps go through the LDS crossbar (__shfl_xor).
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
-  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, true);  // typed: keeps v's known-canonical status
 }
 
 __device__ __forceinline__ void group_minmax(float& mn, float& mx, int span) {

@@ -334,6 +334,14 @@ inline int mov_dpp(int v, int ctrl, int row_mask, int bank_mask, bool bound_ctrl
   return static_cast<int>(static_cast<uint32_t>(w->slot[buf][src]));
 }
 
+inline float update_dpp_f32(float v, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+  int bits;
+  std::memcpy(&bits, &v, 4);
+  bits = mov_dpp(bits, ctrl, row_mask, bank_mask, bound_ctrl);
+  std::memcpy(&v, &bits, 4);
+  return v;
+}
+
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
 
 // v_mfma_f32_32x32x2_f32: A-operand lane l = A[l % 32][l / 32], B-operand lane l
@@ -419,6 +427,7 @@ static inline uint64_t __ballot(bool p) { return hipemu::ballot(p); }
 #define __builtin_amdgcn_readlane(v, l) static_cast<int>(hipemu::readlane_u32(static_cast<uint32_t>(v), (l)))
 #define __builtin_amdgcn_readfirstlane(v) static_cast<int>(hipemu::readfirstlane_u32(static_cast<uint32_t>(v)))
 #define __builtin_amdgcn_mov_dpp(v, ctrl, rm, bm, bc) hipemu::mov_dpp((v), (ctrl), (rm), (bm), (bc))
+#define __builtin_amdgcn_update_dpp(old, v, ctrl, rm, bm, bc) hipemu::update_dpp_f32((v), (ctrl), (rm), (bm), (bc))
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) hipemu::mfma_f32_32x32x2f32((a), (b), (c), (x), (y), (z))
 
 static inline float __fmaf_rn(float a, float b, float c) { return std::fmaf(a, b, c); }
