@@ -21,3 +21,8 @@ def native_batch_norm_backward(grad_out, input, weight, running_mean, running_va
                                train, eps, output_mask):
     return torch.ops.aten.native_batch_norm_backward(grad_out, input, weight, running_mean, running_var,
                                                      save_mean, save_invstd, train, eps, list(output_mask))
+
+
+def _elu_backward_cuda(grad_output, data, alpha):
+    """backward_func_cuda_kernel.cu:6-36: x >= 0 ? grad : alpha * grad * exp(x)."""
+    return torch.where(data >= 0, grad_output, alpha * grad_output * torch.exp(data))

@@ -163,6 +163,38 @@ def act_quantized_relu(input):  # noqa: A002
     return ActQuantizedReLU.apply(input)
 
 
+class ActQuantizedLeakyReLU(torch.autograd.Function):
+    """quantization.cc:87-103."""
+
+    @staticmethod
+    def forward(ctx, input, slope):  # noqa: A002
+        n = input.numel()
+        out = torch.empty_like(input)
+        mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
+        rc = _lib.lib().exact_leaky_relu_fwd_f32(ptr(input), n, float(slope), ptr(out), ptr(mask),
+                                                 _checks.stream_ptr(input))
+        _lib.check(rc, "act_quantized_leaky_relu")
+        ctx.save_for_backward(mask)
+        ctx.slope = float(slope)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (mask,) = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        grad_input = torch.empty_like(grad_output)
+        rc = _lib.lib().exact_leaky_relu_bwd_f32(ptr(grad_output), ptr(mask), grad_output.numel(), ctx.slope,
+                                                 ptr(grad_input), _checks.stream_ptr(grad_output))
+        _lib.check(rc, "act_quantized_leaky_relu backward")
+        return grad_input, None
+
+
+def act_quantized_leaky_relu(input, slope):  # noqa: A002
+    """quantization.cc:105-108."""
+    check_device_tensor(input, "input")
+    return ActQuantizedLeakyReLU.apply(input, slope)
+
+
 class ActQuantizedDropout(torch.autograd.Function):
     """quantization.cc:111-129."""
 

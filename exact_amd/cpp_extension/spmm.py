@@ -1,7 +1,6 @@
 """Stand-in for the reference's `exact.cpp_extension.spmm` module
-(spmm.cc:243-252): spmm_sum_fw/bw and spmm_mean_fw/bw with the reference's
-argument lists.  max/min reductions and gradients with respect to the edge
-values are outside this library's scope and raise.
+(spmm.cc:243-252): spmm_{sum,mean,max,min}_{fw,bw} with the reference's
+argument lists, plus spmm_value_bw (the edge-value gradient).
 """
 from __future__ import annotations
 
@@ -29,7 +28,7 @@ def spmm_csr(rowptr, col, value, mat, reduce):
     """spmm_cuda(rowptr, col, optional_value, mat, reduce) for reduce in
     {sum, mean} (spmm_cuda.cu:106-170)."""
     if reduce not in REDUCE:
-        raise NotImplementedError(f"reduce='{reduce}' is not implemented by this library (sum, mean only)")
+        raise NotImplementedError(f"reduce='{reduce}': use spmm_max_fw / spmm_min_fw for max and min")
     _check_index(rowptr, "rowptr")
     _check_index(col, "col")
     if not _checks.on_device(mat):
@@ -125,36 +124,111 @@ def clear_csc_cache():
     _CSC_CACHE.clear()
 
 
-def _no_value_grad(has_value, value_requires_grad):
-    if has_value and value_requires_grad:
-        raise NotImplementedError(
-            "gradients with respect to the edge values (spmm_value_bw) are not implemented by this library")
+def _same_index_dtype(*ts):
+    wide = torch.int64 if any(t.dtype == torch.int64 for t in ts) else torch.int32
+    return [t.to(wide).contiguous() for t in ts]
+
+
+def spmm_value_bw(row, rowptr, col, mat, grad, reduce):
+    """spmm_value_bw_cuda (spmm_cuda.cu:211-252): gradient with respect to the
+    edge values, out[e] = mat[col[e]] . grad[row[e]] (/ row length for mean)."""
+    if reduce not in REDUCE:
+        raise NotImplementedError(f"reduce='{reduce}'")
+    for t, name in ((row, "row"), (rowptr, "rowptr"), (col, "col")):
+        _check_index(t, name)
+    for t, name in ((mat, "mat"), (grad, "grad")):
+        if not _checks.on_device(t):
+            raise RuntimeError(f"{name} must be CUDA tensor")
+        if t.dim() != 2 or t.dtype != torch.float32:
+            raise RuntimeError(f"The type of {name} is not correct!")
+    row, rowptr, col = _same_index_dtype(row, rowptr, col)
+    mat, grad = mat.contiguous(), grad.contiguous()
+    if mat.shape[1] != grad.shape[1]:
+        raise RuntimeError("Input mismatch")
+    out = torch.zeros(row.numel(), dtype=grad.dtype, device=grad.device)
+    rc = _lib.lib().exact_sddmm_f32(ptr(row), ptr(rowptr), ptr(col), row.element_size(), ptr(mat), ptr(grad),
+                                    row.numel(), mat.shape[1], REDUCE[reduce], ptr(out), _checks.stream_ptr(grad))
+    _lib.check(rc, "spmm_value_bw")
+    return out
 
 
 def spmm_sum_bw(row, rowptr, col, value, colptr, csr2csc, mat, grad_out,
                 has_value, value_requires_grad, mat_requires_grad):
     """spmm.cc:57-79 -> (grad_value, grad_mat)."""
-    _no_value_grad(has_value, value_requires_grad)
+    grad_value = None
+    if has_value and value_requires_grad:
+        grad_value = spmm_value_bw(row, rowptr, col, mat, grad_out, "sum")
     grad_mat = None
     if mat_requires_grad:
         row_csc, val_csc = _csc_operands("sum", row, value, None, csr2csc, has_value, grad_out.dtype)
         grad_mat = spmm_csr(colptr, row_csc, val_csc, grad_out, "sum")
-    return None, grad_mat
+    return grad_value, grad_mat
 
 
 def spmm_mean_bw(row, rowptr, col, value, rowcount, colptr, csr2csc, mat, grad_out,
                  has_value, value_requires_grad, mat_requires_grad):
     """spmm.cc:115-139 -> (grad_value, grad_mat)."""
-    _no_value_grad(has_value, value_requires_grad)
+    grad_value = None
+    if has_value and value_requires_grad:
+        grad_value = spmm_value_bw(row, rowptr, col, mat, grad_out, "mean")
     grad_mat = None
     if mat_requires_grad:
         row_csc, w_csc = _csc_operands("mean", row, value, rowcount, csr2csc, has_value, grad_out.dtype)
         grad_mat = spmm_csr(colptr, row_csc, w_csc, grad_out, "sum")
-    return None, grad_mat
+    return grad_value, grad_mat
 
 
-def _unsupported(*_a, **_k):
-    raise NotImplementedError("max/min aggregation is not implemented by this library (sum, mean only)")
+# ---- max / min aggregation ----------------------------------------------------
+def _spmm_extreme_fw(rowptr, col, value, mat, is_max):
+    """spmm_max_fw / spmm_min_fw (spmm.cc:145-157, 199-212) -> (out, arg_out)."""
+    _check_index(rowptr, "rowptr")
+    _check_index(col, "col")
+    if not _checks.on_device(mat):
+        raise RuntimeError("mat must be CUDA tensor")
+    if mat.dim() != 2 or mat.dtype != torch.float32:
+        raise RuntimeError("The type of mat is not correct!")
+    if value is not None:
+        if value.dim() != 1 or value.size(0) != col.size(0):
+            raise RuntimeError("Input mismatch")
+        value = value.detach().float().contiguous()
+    rowptr, col = _same_index_dtype(rowptr, col)
+    mat = mat.contiguous()
+    M, K = rowptr.numel() - 1, mat.shape[1]
+    out = torch.empty((M, K), dtype=mat.dtype, device=mat.device)
+    arg_out = torch.empty((M, K), dtype=rowptr.dtype, device=mat.device)
+    rc = _lib.lib().exact_spmm_csr_minmax_f32(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat), M,
+                                              mat.shape[0], K, col.numel(), 1 if is_max else 0, ptr(out), ptr(arg_out),
+                                              _checks.stream_ptr(mat))
+    _lib.check(rc, "spmm_max_fw" if is_max else "spmm_min_fw")
+    return out, arg_out
 
 
-spmm_max_fw = spmm_max_bw = spmm_min_fw = spmm_min_bw = _unsupported
+def spmm_max_fw(rowptr, col, value, mat):
+    return _spmm_extreme_fw(rowptr, col, value, mat, True)
+
+
+def spmm_min_fw(rowptr, col, value, mat):
+    return _spmm_extreme_fw(rowptr, col, value, mat, False)
+
+
+def spmm_max_bw(col, value, mat, arg_out, grad_out, has_value, value_requires_grad, mat_requires_grad):
+    """spmm.cc:159-193: route each output gradient back to the entry that won
+    (torch gathers / scatters, as in the reference)."""
+    arg_out = arg_out.long()
+    invalid = arg_out == col.size(0)
+    arg = arg_out.masked_fill(invalid, 0)
+    src = col.long().index_select(0, arg.flatten()).view_as(arg)
+    grad_value = None
+    if has_value and value_requires_grad:
+        picked = mat.gather(-2, src) * grad_out
+        picked.masked_fill_(invalid, 0)
+        grad_value = torch.zeros_like(value).scatter_add_(0, arg.flatten(), picked.flatten())
+    grad_mat = None
+    if mat_requires_grad:
+        contrib = value.detach().index_select(0, arg.flatten()).view_as(arg) * grad_out if has_value else grad_out.clone()
+        contrib.masked_fill_(invalid, 0)
+        grad_mat = torch.zeros_like(mat).scatter_add_(-2, src, contrib)
+    return grad_value, grad_mat
+
+
+spmm_min_bw = spmm_max_bw      # identical routing (spmm.cc:214-241)

@@ -113,6 +113,50 @@ __global__ __launch_bounds__(kBlock) void relu_bwd_kernel(const float* __restric
   }
 }
 
+// LeakyReLU with the same 1-bit mask (quantization_cuda_kernel.cu:339-371, 395-412):
+// y = x > 0 ? x : x * slope; dx = bit ? dy : dy * slope.
+template <bool VEC4>
+__global__ __launch_bounds__(kBlock) void leaky_relu_fwd_kernel(const float* __restrict__ x, int64_t n, float slope,
+                                                                float* __restrict__ y,
+                                                                uint32_t* __restrict__ mask) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
+    const int nv = valid_in_quad(quad, n);
+    float v[4];
+    uint32_t nibble = 0;
+    if (nv > 0) {
+      load4<VEC4>(x + quad * 4, nv, v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool bit = v[i] > 0.f;
+        v[i] = bit ? v[i] : v[i] * slope;
+        nibble |= static_cast<uint32_t>(bit && i < nv) << i;
+      }
+      store4<VEC4>(y + quad * 4, nv, v);
+    }
+    store_mask_nibble(nibble, quad, n, mask);
+  }
+}
+
+template <bool VEC4>
+__global__ __launch_bounds__(kBlock) void leaky_relu_bwd_kernel(const float* __restrict__ dy,
+                                                                const uint32_t* __restrict__ mask, int64_t n,
+                                                                float slope, float* __restrict__ dx) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
+    const int nv = valid_in_quad(quad, n);
+    if (nv == 0) continue;
+    float v[4];
+    load4<VEC4>(dy + quad * 4, nv, v);
+    const uint32_t nibble = load_mask_nibble(mask, quad);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = ((nibble >> i) & 1u) ? v[i] : v[i] * slope;
+    store4<VEC4>(dx + quad * 4, nv, v);
+  }
+}
+
 template <bool VEC4, bool NOISE_IN>
 __global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ noise,
@@ -214,6 +258,31 @@ int exact_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float* 
     hipLaunchKernelGGL((relu_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
   else
     hipLaunchKernelGGL((relu_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
+  return launch_status();
+}
+
+int exact_leaky_relu_fwd_f32(const float* x, int64_t n, float slope, float* y, uint32_t* mask, void* stream) {
+  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+  if (n == 0) return EXACT_OK;
+  if (!x || !y || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (aligned16(x) && aligned16(y))
+    hipLaunchKernelGGL((leaky_relu_fwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, x, n, slope, y, mask);
+  else
+    hipLaunchKernelGGL((leaky_relu_fwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, x, n, slope, y, mask);
+  return launch_status();
+}
+
+int exact_leaky_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float slope, float* dx,
+                             void* stream) {
+  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+  if (n == 0) return EXACT_OK;
+  if (!dy || !dx || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (aligned16(dy) && aligned16(dx))
+    hipLaunchKernelGGL((leaky_relu_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, slope, dx);
+  else
+    hipLaunchKernelGGL((leaky_relu_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, slope, dx);
   return launch_status();
 }
 

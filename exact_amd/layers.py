@@ -9,7 +9,7 @@ from torch.nn import Parameter
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCNConv, SAGEConv, glorot
-from .ops import input2rp, qbatch_norm, qlinear, quantize_activation
+from .ops import input2rp, qbatch_norm, qelu, qlinear, quantize_activation
 from .qsheme import QScheme
 from .spmm import QMatmul
 
@@ -114,6 +114,30 @@ class QReLU(torch.nn.Module):
         if self.training:
             return ext_quantization.act_quantized_relu(input)
         return F.relu(input)
+
+
+class QLeakyReLU(torch.nn.Module):
+    """layers.py:295-301 of the reference (compressed in train and eval alike)."""
+
+    def __init__(self, negative_slope, inplace=False):
+        super().__init__()
+        self.negative_slope = negative_slope
+
+    def forward(self, input):  # noqa: A002
+        return ext_quantization.act_quantized_leaky_relu(input, self.negative_slope)
+
+
+class QELU(torch.nn.Module):
+    """layers.py:304-313 of the reference."""
+
+    def __init__(self, alpha, inplace=False):
+        super().__init__()
+        self.alpha = alpha
+
+    def forward(self, input):  # noqa: A002
+        if self.training:
+            return qelu.apply(input, self.alpha)
+        return F.elu(input, self.alpha)
 
 
 class QDropout(torch.nn.Module):

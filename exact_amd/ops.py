@@ -307,3 +307,80 @@ class qspmm_mean(Function):
                                                  grad_outputs.contiguous(), has_value, value_requires_grad,
                                                  mat_requires_grad)
         return None, None, None, grad_value, None, None, None, None, grad_mat, None, None, None
+
+
+class qelu(Function):
+    """ELU that keeps its input compressed (reference ops.py:182-204)."""
+
+    @staticmethod
+    def forward(ctx, input, alpha, scheme=None):  # noqa: A002
+        ctx.kept = CompressedActivation.compress(input, scheme, project=False)
+        ctx.alpha = alpha
+        empty_cache(config.empty_cache_threshold)
+        return F.elu(input, alpha)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x_hat = ctx.kept.restore()
+        ctx.kept = None
+        empty_cache(config.empty_cache_threshold)
+        return ext_backward_func._elu_backward_cuda(grad_output, x_hat, ctx.alpha), None, None
+
+
+def _extreme_forward(ctx, is_max, rowptr, col, value, has_value, other, quantized, scheme):
+    """Shared forward of qspmm_max / qspmm_min (reference ops.py:374-436).  The
+    dense operand is read again in backward only for the edge-value gradient,
+    so it is compressed and kept only then (or when the caller supplies it)."""
+    fw = spmm.spmm_max_fw if is_max else spmm.spmm_min_fw
+    output, arg_out = fw(rowptr, col, value, other)
+    value_requires_grad = bool(has_value and value.requires_grad)
+    if quantized is not None:
+        assert isinstance(quantized, tuple)
+        kept = CompressedActivation(quantized, None, other.shape, other.shape)
+    elif value_requires_grad or config.keep_unused_spmm_operand:
+        kept = CompressedActivation.compress(other, scheme, project=False)
+    else:
+        kept = None
+    empty_cache(config.empty_cache_threshold)
+    ctx.kept, ctx.graph, ctx.operand_shape = kept, (col, value, arg_out), other.shape
+    ctx.flags = (has_value, value_requires_grad, other.requires_grad)
+    ctx.mark_non_differentiable(arg_out)
+    return output
+
+
+def _extreme_backward(ctx, grad_outputs):
+    col, value, arg_out = ctx.graph
+    has_value, value_requires_grad, mat_requires_grad = ctx.flags
+    if value_requires_grad:
+        other = ctx.kept.restore()
+    else:  # only the operand's shape is needed to size grad_mat
+        other = grad_outputs.new_empty(ctx.operand_shape)
+    ctx.kept = None
+    empty_cache(config.empty_cache_threshold)
+    grad_value, grad_mat = spmm.spmm_max_bw(col, value, other, arg_out, grad_outputs.contiguous(), has_value,
+                                            value_requires_grad, mat_requires_grad)
+    return None, None, grad_value, None, grad_mat, None, None, None
+
+
+class qspmm_max(Function):
+    """out = max over the entries of each row of val * X[col]  (reference ops.py:374-403)."""
+
+    @staticmethod
+    def forward(ctx, rowptr, col, value, has_value, other, quantized=None, randmat=None, scheme=None):
+        return _extreme_forward(ctx, True, rowptr, col, value, has_value, other, quantized, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        return _extreme_backward(ctx, grad_outputs)
+
+
+class qspmm_min(Function):
+    """Reference ops.py:406-436; gradients are routed as for max (spmm.cc:214-241)."""
+
+    @staticmethod
+    def forward(ctx, rowptr, col, value, has_value, other, quantized=None, randmat=None, scheme=None):
+        return _extreme_forward(ctx, False, rowptr, col, value, has_value, other, quantized, scheme)
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        return _extreme_backward(ctx, grad_outputs)

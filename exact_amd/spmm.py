@@ -4,7 +4,7 @@ operand (anything exposing .csr() and .storage with the cached vectors)."""
 import torch
 
 from .conf import config
-from .ops import qspmm_mean, qspmm_sum
+from .ops import qspmm_max, qspmm_mean, qspmm_min, qspmm_sum
 from .qsheme import QScheme
 
 
@@ -26,8 +26,10 @@ def _dispatch(src, other, reduce, quantized, randmat, scheme):
             row, rowcount, csr2csc, colptr = st.row(), st.rowcount(), st.csr2csc(), st.colptr()
         return qspmm_mean.apply(row, rowptr, col, value, rowcount, colptr, csr2csc, has_value, other,
                                 quantized, randmat, scheme)
-    if reduce in ("min", "max"):
-        raise NotImplementedError("min/max aggregation is not implemented by this library (sum, mean only)")
+    if reduce == "max":
+        return qspmm_max.apply(rowptr, col, value, has_value, other, quantized, randmat, scheme)
+    if reduce == "min":
+        return qspmm_min.apply(rowptr, col, value, has_value, other, quantized, randmat, scheme)
     raise ValueError(reduce)
 
 

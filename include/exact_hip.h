@@ -122,6 +122,34 @@ int exact_spmm_csr_f32(const void *rowptr, const void *col, const float *val,
                        int idx_bytes, const float *X, int64_t M, int64_t n_cols,
                        int64_t K, int64_t nnz, int reduce, float *out, void *stream);
 
+/* Max / min aggregation: out[r, k] = max (is_max != 0) or min over the entries
+ * e of row r of val[e] * X[col[e], k]; arg_out[r, k] (same index type as
+ * rowptr / col, [M, K]) = the first entry index attaining it; rows without
+ * entries give out = 0 and arg_out = nnz.  Replaces spmm_cuda(..., "max" |
+ * "min") as called by spmm_max_fw / spmm_min_fw (spmm.cc:145-157, 199-212;
+ * kernel spmm_cuda.cu:27-104 with Reducer<MAX|MIN> reducer.cuh:43-85). */
+int exact_spmm_csr_minmax_f32(const void *rowptr, const void *col, const float *val,
+                              int idx_bytes, const float *X, int64_t M, int64_t n_cols,
+                              int64_t K, int64_t nnz, int is_max, float *out,
+                              void *arg_out, void *stream);
+
+/* Gradient with respect to the edge values: out[e] = sum_k mat[col[e], k] *
+ * grad[row[e], k], divided by max(length of row[e], 1) for EXACT_REDUCE_MEAN.
+ * row is the COO row index of every entry.  Replaces spmm_value_bw_cuda
+ * (spmm_cuda.cu:172-252) as called by spmm_sum_bw / spmm_mean_bw
+ * (spmm.cc:65-67, 123-125). */
+int exact_sddmm_f32(const void *row, const void *rowptr, const void *col, int idx_bytes,
+                    const float *mat, const float *grad, int64_t nnz, int64_t K,
+                    int reduce, float *out, void *stream);
+
+/* LeakyReLU with the 1-bit mask of a13: y = x > 0 ? x : x * slope;
+ * dx = bit ? dy : dy * slope.  Replaces act_quantized_leakyrelu_forward_cuda /
+ * _backward_cuda (quantization_cuda_kernel.cu:339-435). */
+int exact_leaky_relu_fwd_f32(const float *x, int64_t n, float slope, float *y,
+                             uint32_t *mask, void *stream);
+int exact_leaky_relu_bwd_f32(const float *dy, const uint32_t *mask, int64_t n,
+                             float slope, float *dx, void *stream);
+
 /* a7. Random projection: out[N, k] = X[N, D] . R[D, k]  (input2rp, ops.py:107-118)
  * and back: out[N, D] = Xr[N, k] . R[D, k]^T  (rp2input, ops.py:121-125).
  * fp32 in, fp32 accumulate on the matrix cores. */

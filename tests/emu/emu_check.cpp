@@ -179,6 +179,81 @@ static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
   CHECK(worst <= 2e-5 * scale, "rp bwd differs N=%ld D=%ld k=%ld: %g of %g", (long)N, (long)D, (long)k, worst, scale);
 }
 
+// LeakyReLU mask, max / min aggregation and the edge-value gradient, against
+// straight loops written here (the Python oracle for them is
+// oracle/exact_oracle_extra.py, checked by tests/test_more_ops.py).
+static void check_extra(int64_t M, int64_t ncols, int64_t K, double avg, std::mt19937& rng) {
+  const Csr g = powerlaw(M, ncols, avg, 0, rng);
+  const int64_t nnz = (int64_t)g.col.size();
+  std::normal_distribution<float> nd(0.f, 1.f);
+  Buf<float> X(ncols * K), grad(M * K), out(M * K), val(nnz), ev(nnz);
+  Buf<int64_t> rp64(M + 1), col64(nnz), row64(nnz), arg64(M * K);
+  Buf<int32_t> rp32(M + 1), col32(nnz), row32(nnz), arg32(M * K);
+  for (int64_t i = 0; i < ncols * K; ++i) X[i] = nd(rng);
+  for (int64_t i = 0; i < M * K; ++i) grad[i] = nd(rng);
+  for (int64_t i = 0; i <= M; ++i) { rp64[i] = g.rowptr[i]; rp32[i] = (int32_t)g.rowptr[i]; }
+  for (int64_t r = 0; r < M; ++r)
+    for (int64_t e = g.rowptr[r]; e < g.rowptr[r + 1]; ++e) { row64[e] = r; row32[e] = (int32_t)r; }
+  for (int64_t i = 0; i < nnz; ++i) { col64[i] = g.col[i]; col32[i] = (int32_t)g.col[i]; val[i] = g.val[i]; }
+  for (int is_max = 0; is_max < 2; ++is_max)
+    for (int valued = 0; valued < 2; ++valued)
+      for (int wide = 0; wide < 2; ++wide) {
+        const float* v = valued ? val.p : nullptr;
+        const int rc = wide ? exact_spmm_csr_minmax_f32(rp64.p, col64.p, v, 8, X.p, M, ncols, K, nnz, is_max, out.p, arg64.p, nullptr)
+                            : exact_spmm_csr_minmax_f32(rp32.p, col32.p, v, 4, X.p, M, ncols, K, nnz, is_max, out.p, arg32.p, nullptr);
+        CHECK(rc == 0, "minmax rc=%d", rc);
+        int64_t bad = 0;
+        for (int64_t r = 0; r < M; ++r)
+          for (int64_t k = 0; k < K; ++k) {
+            float best = 0.f;
+            int64_t arg = nnz;
+            for (int64_t e = g.rowptr[r]; e < g.rowptr[r + 1]; ++e) {
+              const float t = valued ? g.val[e] * X[g.col[e] * K + k] : X[g.col[e] * K + k];
+              if (arg == nnz || (is_max ? t > best : t < best)) { best = t; arg = e; }
+            }
+            const int64_t got = wide ? arg64[r * K + k] : (int64_t)arg32[r * K + k];
+            bad += (out[r * K + k] != best) || (got != arg);
+          }
+        CHECK(bad == 0, "minmax differs M=%ld K=%ld max=%d valued=%d wide=%d: %ld cells", (long)M, (long)K, is_max, valued, wide, (long)bad);
+      }
+  for (int reduce = 0; reduce < 2; ++reduce)
+    for (int wide = 0; wide < 2; ++wide) {
+      const int rc = wide ? exact_sddmm_f32(row64.p, rp64.p, col64.p, 8, X.p, grad.p, nnz, K, reduce, ev.p, nullptr)
+                          : exact_sddmm_f32(row32.p, rp32.p, col32.p, 4, X.p, grad.p, nnz, K, reduce, ev.p, nullptr);
+      CHECK(rc == 0, "sddmm rc=%d", rc);
+      double worst = 0, scale = 1e-30;
+      for (int64_t r = 0; r < M; ++r)
+        for (int64_t e = g.rowptr[r]; e < g.rowptr[r + 1]; ++e) {
+          double acc = 0;
+          for (int64_t k = 0; k < K; ++k) acc += (double)X[g.col[e] * K + k] * (double)grad[r * K + k];
+          if (reduce) acc /= (double)std::max<int64_t>(g.rowptr[r + 1] - g.rowptr[r], 1);
+          scale = std::max(scale, std::fabs(acc));
+          worst = std::max(worst, std::fabs(acc - (double)ev[e]));
+        }
+      CHECK(worst <= 1e-5 * scale, "sddmm differs M=%ld K=%ld reduce=%d wide=%d: %g of %g", (long)M, (long)K, reduce, wide, worst, scale);
+    }
+}
+
+static void check_leaky(int64_t n, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 1.f);
+  const int64_t words = (n + 31) / 32;
+  Buf<float> x(n), g(n), y(n), dx(n);
+  Buf<uint32_t> m(words);
+  for (int64_t i = 0; i < n; ++i) { x[i] = nd(rng); g[i] = nd(rng); }
+  const float slope = 0.2f;
+  CHECK(exact_leaky_relu_fwd_f32(x.p, n, slope, y.p, m.p, nullptr) == 0, "leaky rc");
+  CHECK(exact_leaky_relu_bwd_f32(g.p, m.p, n, slope, dx.p, nullptr) == 0, "leaky bwd rc");
+  int64_t bad = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const bool pos = x[i] > 0.f;
+    bad += y[i] != (pos ? x[i] : x[i] * slope);
+    bad += ((m[i / 32] >> (i % 32)) & 1u) != (pos ? 1u : 0u);
+    bad += dx[i] != (pos ? g[i] : g[i] * slope);
+  }
+  for (int64_t i = n; i < words * 32; ++i) bad += (m[i / 32] >> (i % 32)) & 1u;  // tail bits are written as 0
+  CHECK(bad == 0, "leaky relu differs n=%ld: %ld", (long)n, (long)bad);
+}
+
 int main(int argc, char** argv) {
   std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
@@ -204,6 +279,14 @@ int main(int argc, char** argv) {
                             {64, 128, 64}, {77, 50, 15}, {130, 7, 4}, {100, 256, 126}, {33, 256, 128}};
   for (auto& s : rps) check_rp(s[0], s[1], s[2], rng);
   std::printf("rp shapes ok (failures so far %d)\n", g_fail);
+  for (int64_t n : {1, 3, 31, 32, 33, 255, 257, 1000, 2049, 4101, 50001}) check_leaky(n, rng);
+  check_extra(120, 120, 256, 6, rng);
+  check_extra(80, 50, 40, 5, rng);
+  check_extra(60, 60, 602, 4, rng);
+  check_extra(70, 33, 7, 8, rng);
+  check_extra(40, 40, 1, 3, rng);
+  check_extra(50, 50, 1000, 3, rng);
+  std::printf("leaky / minmax / sddmm ok (failures so far %d)\n", g_fail);
   if (mode == "full") {
     for (int bits : {1, 2, 4, 8}) check_quant(169343, 256, bits, bits == 2, rng);
     std::printf("full-size quant ok (failures so far %d)\n", g_fail);

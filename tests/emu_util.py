@@ -165,3 +165,47 @@ def rp_bwd(Xr, R, guard=16):
     assert emu().exact_rp_bwd_f32(p(Xr), p(R), N, D, k, p(out), None) == 0
     assert (out[N * D:] == np.float32(-777.0)).all()
     return out[:N * D].reshape(N, D)
+
+
+def leaky_relu_fwd(x, slope, guard=8):
+    x = f32(x).reshape(-1)
+    n = x.size
+    y = np.full(n + guard, np.float32(7.0), np.float32)
+    words = (n + 31) // 32
+    mask = np.full(words + guard, 0x5A5A5A5A, np.uint32)
+    assert emu().exact_leaky_relu_fwd_f32(p(x), n, slope, p(y), p(mask), None) == 0
+    assert (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
+    return y[:n], mask[:words]
+
+
+def leaky_relu_bwd(dy, mask, slope):
+    dy = f32(dy).reshape(-1)
+    dx = np.zeros_like(dy)
+    assert emu().exact_leaky_relu_bwd_f32(p(dy), p(np.ascontiguousarray(mask, np.uint32)), dy.size, slope, p(dx), None) == 0
+    return dx
+
+
+def spmm_minmax(rowptr, col, val, X, is_max, idx=np.int64, guard=16):
+    rowptr = np.ascontiguousarray(rowptr, dtype=idx)
+    col = np.ascontiguousarray(col, dtype=idx)
+    X = f32(X)
+    val = None if val is None else f32(val)
+    M, K = rowptr.size - 1, X.shape[1]
+    out = np.full(M * K + guard, np.float32(-777.0), np.float32)
+    arg = np.full(M * K + guard, -5, idx)
+    rc = emu().exact_spmm_csr_minmax_f32(p(rowptr), p(col), p(val), rowptr.itemsize, p(X), M, X.shape[0], K, col.size,
+                                         1 if is_max else 0, p(out), p(arg), None)
+    assert rc == 0, rc
+    assert (out[M * K:] == np.float32(-777.0)).all() and (arg[M * K:] == -5).all()
+    return out[:M * K].reshape(M, K), arg[:M * K].reshape(M, K)
+
+
+def sddmm(row, rowptr, col, mat, grad, reduce, idx=np.int64, guard=8):
+    row, rowptr, col = (np.ascontiguousarray(a, dtype=idx) for a in (row, rowptr, col))
+    mat, grad = f32(mat), f32(grad)
+    out = np.full(row.size + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_sddmm_f32(p(row), p(rowptr), p(col), row.itemsize, p(mat), p(grad), row.size, mat.shape[1],
+                               1 if reduce == "mean" else 0, p(out), None)
+    assert rc == 0, rc
+    assert (out[row.size:] == np.float32(-777.0)).all()
+    return out[:row.size]

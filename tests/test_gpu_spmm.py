@@ -145,5 +145,5 @@ def test_gcn_norm_and_errors(cuda):
         ext_spmm.spmm_sum_fw(None, rowptr, col, value, None, None, torch.randn(500, 8, device=cuda, requires_grad=True))
     with pytest.raises(RuntimeError, match="Input mismatch"):
         ext_spmm.spmm_csr(rowptr, col, value[:-1], torch.randn(500, 8, device=cuda), "sum")
-    with pytest.raises(NotImplementedError):
-        qmatmul(adj, torch.randn(500, 8, device=cuda), "max")
+    with pytest.raises(ValueError):
+        qmatmul(adj, torch.randn(500, 8, device=cuda), "mul")

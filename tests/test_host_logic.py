@@ -61,10 +61,10 @@ def test_shims_reject_host_tensors_with_the_reference_messages():
         ops.quantize_activation(x, None)
     with pytest.raises(RuntimeError, match="must be CUDA tensor"):
         ext_spmm.spmm_csr(torch.zeros(9, dtype=torch.long), torch.zeros(0, dtype=torch.long), None, x, "sum")
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError, match="spmm_max_fw"):
         ext_spmm.spmm_csr(torch.zeros(9, dtype=torch.long), torch.zeros(0, dtype=torch.long), None, x, "max")
-    with pytest.raises(NotImplementedError):
-        ext_spmm.spmm_max_fw()
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        ext_spmm.spmm_max_fw(torch.zeros(9, dtype=torch.long), torch.zeros(0, dtype=torch.long), None, x)
 
 
 def test_sparse_tensor_matches_scipy():
