@@ -70,6 +70,25 @@ def cpu_baseline(x_host, step_bytes, seed, min_seconds=10.0, max_passes=20):
             "seconds_per_step": cpu_s, "host_cpus": os.cpu_count()}
 
 
+def run_extras(rows, cols, scale, timeout_s=420):
+    """The secondary measurements (mask / projection / SpMM kernels, epochs/s of
+    the three model configurations) in a child process: whatever happens there,
+    the headline figures measured in this process are still printed."""
+    import subprocess
+    cmd = [sys.executable, "-m", "exact_amd.benchmarks", "extras", "--rows", str(rows), "--cols", str(cols),
+           "--scale", str(scale)]
+    try:
+        res = subprocess.run(cmd, cwd=ROOT, stdout=subprocess.PIPE, timeout=timeout_s, text=True)
+    except subprocess.TimeoutExpired:
+        return {"error": f"extras child exceeded {timeout_s} s"}
+    except OSError as e:
+        return {"error": f"extras child could not start: {e}"}
+    lines = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+    if res.returncode != 0 or not lines:
+        return {"error": f"extras child exited with {res.returncode}"}
+    return json.loads(lines[-1])
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -79,6 +98,7 @@ def main(argv=None):
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--extras-scale", type=float, default=1.0, help=argparse.SUPPRESS)
+    ap.add_argument("--extras-in-process", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args(argv)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus must be 1 (the path has no multi-GPU code; "
@@ -91,8 +111,7 @@ def main(argv=None):
     L = _lib.lib()  # raises if the HIP library is missing: there is no fallback
     dev = benchmarks.bench_device()
     N, G = args.rows, N_COLS
-    gen = torch.Generator(device=dev).manual_seed(1234)
-    x = torch.randn((N, G), generator=gen, device=dev, dtype=torch.float32)
+    x = benchmarks.headline_input(N, G, dev)
     out = torch.empty_like(x)
     sp = _checks.stream_ptr(x)
     packed = {b: torch.empty(int(L.exact_packed_nbytes(N, G, b)), dtype=torch.int8, device=dev) for b in BITS}
@@ -161,13 +180,14 @@ def main(argv=None):
         except Exception as e:  # noqa: BLE001
             log(f"cpu baseline failed: {type(e).__name__}: {e}")
 
-    extras = {}
-    if not args.no_extras:
-        try:
-            extras = benchmarks.run(x, log, scale=args.extras_scale)
-        except Exception as e:  # noqa: BLE001 -- extras never invalidate the headline line
-            log(f"extras failed: {type(e).__name__}: {e}")
-            extras = {"error": f"{type(e).__name__}: {e}"}
+    if args.no_extras:
+        extras = {}
+    elif args.extras_in_process:
+        extras = benchmarks.run(x, log, scale=args.extras_scale)
+    else:
+        extras = run_extras(N, G, args.extras_scale)
+    if "error" in extras:
+        log(f"extras: {extras['error']}")
 
     result = {
         "metric": "pack+unpack GB/s (% HBM peak); INT2 GCN/SAGE full-batch epochs/s",

@@ -8,6 +8,7 @@ with HIP events on the stream the kernels are launched on.
 """
 from __future__ import annotations
 
+import sys
 import time
 
 import torch
@@ -271,6 +272,33 @@ def run(x, log, budget_s=240.0, epoch_configs=("cfg3_gcn_int2", "cfg4_sage_int2_
     return out
 
 
+def headline_input(rows, cols, device):
+    """The benchmark activation: fp32 [rows, cols] ~ N(0,1), fixed seed."""
+    gen = torch.Generator(device=device).manual_seed(1234)
+    return torch.randn((rows, cols), generator=gen, device=device, dtype=torch.float32)
+
+
+def _extras_main(argv):
+    """`python -m exact_amd.benchmarks extras`: run() in a process of its own
+    and print its result as one JSON line (bench.py starts it as a child, so
+    that nothing that happens here can take the headline figure with it)."""
+    import argparse
+    import json
+    ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks extras")
+    ap.add_argument("--rows", type=int, default=169343)
+    ap.add_argument("--cols", type=int, default=256)
+    ap.add_argument("--scale", type=float, default=1.0)
+    ap.add_argument("--budget", type=float, default=240.0)
+    args = ap.parse_args(argv)
+
+    def log(*a):
+        print(*a, file=sys.stderr, flush=True)
+
+    dev = bench_device()
+    x = headline_input(args.rows, args.cols, dev)
+    print(json.dumps(run(x, log, budget_s=args.budget, scale=args.scale)), flush=True)
+
+
 def _profile_target(argv=None):
     """One kernel in a loop, as the target of `rocprofv3 --kernel-trace --stats` /
     `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
@@ -284,6 +312,10 @@ def _profile_target(argv=None):
 
     from . import _lib
     from .cpp_extension import _checks
+    if argv is None:
+        argv = sys.argv[1:]
+    if argv and argv[0] == "extras":
+        return _extras_main(argv[1:])
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
     ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "rp_fwd", "rp_bwd", "spmm", "copy"])
     ap.add_argument("--bits", type=int, default=2)

@@ -79,7 +79,7 @@ def test_bench_py_emits_the_contract_line(cpu_harness, capsys):
     bench = importlib.import_module("bench")
     import bench as b2
     b2.cpu_baseline.__defaults__ = (0.2, 1)
-    bench.main(["--rows", "203", "--steps", "2", "--warmup", "1", "--extras-scale", "0.0005"])
+    bench.main(["--rows", "203", "--steps", "2", "--warmup", "1", "--extras-scale", "0.0005", "--extras-in-process"])
     lines = [l for l in capsys.readouterr().out.splitlines() if l.strip()]
     assert len(lines) == 1
     r = json.loads(lines[0])
@@ -92,3 +92,32 @@ def test_bench_py_emits_the_contract_line(cpu_harness, capsys):
     assert len(r["kernels"]) == 8 and set(r["epochs_per_s"]) == set(bm.EPOCH_CONFIGS)
     with pytest.raises(SystemExit):
         bench.main(["--gpus", "2"])
+
+
+def test_extras_entry_point_prints_one_json_line(cpu_harness, capsys, monkeypatch):
+    """`python -m exact_amd.benchmarks extras` (the child bench.py starts)."""
+    import json
+    monkeypatch.setattr(bm, "run", lambda x, log, budget_s, scale: {"rows": x.shape[0], "scale": scale, "b": budget_s})
+    bm._profile_target(["extras", "--rows", "65", "--cols", "64", "--scale", "0.5", "--budget", "3"])
+    lines = [l for l in capsys.readouterr().out.splitlines() if l.strip()]
+    assert len(lines) == 1 and json.loads(lines[0]) == {"rows": 65, "scale": 0.5, "b": 3.0}
+
+
+def test_failed_extras_child_leaves_an_error_entry(monkeypatch):
+    import os
+    import subprocess
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+
+    class Done:
+        returncode, stdout = -6, "progress\n"
+    monkeypatch.setattr(subprocess, "run", lambda *a, **k: Done())
+    assert "exited with -6" in bench.run_extras(10, 8, 1.0)["error"]
+    Done.returncode, Done.stdout = 0, 'noise\n{"kernels": {}}\n'
+    assert bench.run_extras(10, 8, 1.0) == {"kernels": {}}
+
+    def boom(*a, **k):
+        raise subprocess.TimeoutExpired(a[0], 1)
+    monkeypatch.setattr(subprocess, "run", boom)
+    assert "exceeded" in bench.run_extras(10, 8, 1.0)["error"]
