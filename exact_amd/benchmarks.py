@@ -115,6 +115,16 @@ def kernel_extras(x, log):
         t = event_time(lambda: torch.autograd.grad(yd, xr, gy, retain_graph=True))
         out["dropout_bwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
         del y, yd, gy, xr
+        # --- fused epilogues: ReLU -> dropout (-> INT2 quantise + pack) in one pass --
+        t = event_time(lambda: extq.relu_dropout_fwd(x, 0.5))
+        out["relu_dropout_fwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes,
+                                   "replaces_us": out["relu_fwd"]["us"] + out["dropout_fwd"]["us"]}
+        if extq.fusable_width(G):
+            fused_bytes = mask_bytes + (2 * n) // 8 + 4 * N
+            t = event_time(lambda: extq.relu_dropout_minmax_pack(x, 0.5, 2))
+            t_pack = event_time(lambda: extq.minmax_pack(x, 2))
+            out["relu_dropout_pack_int2"] = {"us": t * 1e6, "GB/s": fused_bytes / t / 1e9, "algo_bytes": fused_bytes,
+                                             "replaces_us": out["relu_fwd"]["us"] + out["dropout_fwd"]["us"] + t_pack * 1e6}
         # --- random projection 256 -> 32 (kept_frac 0.125), Gaussian N(0, 1/k) --
         k = int(0.125 * G + 0.999)
         R = torch.randn(G, k, device=x.device) / k ** 0.5

@@ -43,6 +43,10 @@ _EXTRA_FIELDS = {
     # SpMM although backward reads it only for edge-value gradients; set this to
     # reproduce that memory behaviour.  Results do not depend on it.
     "keep_unused_spmm_operand": False,
+    # ReLU -> dropout -> (quantise for the next layer) as one pass where the
+    # model offers the pair as one module (QReLUDropout).  Results are
+    # bit-identical to the separate layers; False runs them separately.
+    "fuse_epilogue": True,
 }
 
 

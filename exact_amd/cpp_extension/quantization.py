@@ -233,3 +233,58 @@ def act_quantized_dropout(input, p, train):  # noqa: A002
     if not train:
         return input                      # quantization.cc:115-117
     return ActQuantizedDropout.apply(input, p, train)
+
+
+# ---- fused epilogues (no counterpart module function in the reference) -------
+def fusable_width(G: int) -> bool:
+    """Row widths the one-pass ReLU + dropout + quantise kernel takes."""
+    return G > 0 and G % 8 == 0 and G <= 1024
+
+
+def relu_dropout_fwd(input, p):  # noqa: A002
+    """dropout(relu(input)) in one pass -> (output, joint 1-bit mask); the
+    gradient of the pair is dropout_bwd on that mask."""
+    check_device_tensor(input, "input")
+    n = input.numel()
+    out = torch.empty_like(input)
+    mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
+    noise, seed, offset = _noise_for(input.shape, input.device)
+    rc = _lib.lib().exact_relu_dropout_fwd_f32(ptr(input), ptr(noise), seed, offset, float(p), n, ptr(out), ptr(mask),
+                                               _checks.stream_ptr(input))
+    _lib.check(rc, "relu_dropout")
+    return out, mask
+
+
+def relu_dropout_minmax_pack(input, p, bits):  # noqa: A002
+    """dropout(relu(input)) and minmax_pack of the result in one pass over
+    input[N, G] -> (output, mask, packed int8, scale bf16, min bf16).  Draws
+    the dropout noise first, then the quantiser's, as the separate calls do."""
+    check_device_tensor(input, "input", 2)
+    _check_bits(bits)
+    N, G = input.shape
+    if not fusable_width(G):
+        raise RuntimeError("relu_dropout_minmax_pack needs a row width that is a multiple of 8 and at most 1024")
+    dev = input.device
+    out = torch.empty_like(input)
+    mask = torch.empty(mask_nwords(N * G), dtype=torch.int32, device=dev)
+    packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=dev)
+    scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    act_noise, act_seed, act_offset = _noise_for(input.shape, dev)
+    noise, seed, offset = _noise_for(input.shape, dev)
+    rc = _lib.lib().exact_relu_dropout_minmax_pack_f32(
+        ptr(input), float(p), ptr(act_noise), act_seed, act_offset, ptr(noise), seed, offset, N, G, bits,
+        ptr(out), ptr(mask), ptr(packed), None, None, ptr(scale_bf), ptr(min_bf), _checks.stream_ptr(input))
+    _lib.check(rc, "relu_dropout_minmax_pack")
+    return out, mask, packed, scale_bf, min_bf
+
+
+def dropout_bwd(grad_output, mask, p):
+    """dx = bit ? dy / (1 - p) : 0 (quantization_cuda_kernel.cu:565-569)."""
+    grad_output = grad_output.contiguous()
+    check_device_tensor(grad_output, "grad_output")
+    grad_input = torch.empty_like(grad_output)
+    rc = _lib.lib().exact_dropout_bwd_f32(ptr(grad_output), ptr(mask), float(p), grad_output.numel(),
+                                          ptr(grad_input), _checks.stream_ptr(grad_output))
+    _lib.check(rc, "dropout backward")
+    return grad_input

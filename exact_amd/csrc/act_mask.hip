@@ -157,7 +157,10 @@ __global__ __launch_bounds__(kBlock) void leaky_relu_bwd_kernel(const float* __r
   }
 }
 
-template <bool VEC4, bool NOISE_IN>
+// RELU: the input first goes through ReLU and the mask bit is (x > 0) && keep --
+// ReLU followed by dropout in one pass, with one mask for the pair (the
+// backward of the pair is dx = bit ? dy / (1 - p) : 0, i.e. dropout_bwd_kernel).
+template <bool VEC4, bool NOISE_IN, bool RELU>
 __global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ noise,
                                                              uint32_t seed_lo, uint32_t seed_hi,
@@ -193,12 +196,14 @@ __global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const float* __rest
       if constexpr (NOISE_IN) load4<VEC4>(noise + quad * 4, nv, u[h]);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const bool keep = u[h][i] > p;  // quantization_cuda_kernel.cu:465-468
+        const bool pos = !RELU || v[i] > 0.f;  // :252-257
+        const bool keep = u[h][i] > p;         // :465-468
         const float kf = keep ? 1.f : 0.f;
-        float r = v[i] * kf;  // :490, left to right
+        float r = pos ? v[i] : 0.f;
+        r = r * kf;  // :490, left to right
         r = r * pinv;
         v[i] = r;
-        nibble |= static_cast<uint32_t>(keep && i < nv) << i;
+        nibble |= static_cast<uint32_t>(pos && keep && i < nv) << i;
       }
       store4<VEC4>(y + quad * 4, nv, v);
     }
@@ -234,6 +239,30 @@ static dim3 tile_grid(int64_t n) {
 }  // namespace exact
 
 using namespace exact;
+
+template <bool RELU>
+static int dropout_forward(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p, int64_t n,
+                           float* y, uint32_t* mask, void* stream) {
+  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+  if (!(p >= 0.f && p < 1.f)) return EXACT_E_ARG;
+  if (n == 0) return EXACT_OK;
+  if (!x || !y || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // quantization_cuda_kernel.cu:456: float pinv = 1. / (1. - p), evaluated in double
+  const float pinv = static_cast<float>(1.0 / (1.0 - static_cast<double>(p)));
+  const uint32_t sl = static_cast<uint32_t>(seed), sh = static_cast<uint32_t>(seed >> 32);
+  const uint32_t ol = static_cast<uint32_t>(offset), oh = static_cast<uint32_t>(offset >> 32);
+  const bool v4 = aligned16(x) && aligned16(y) && (!noise || aligned16(noise));
+  const dim3 grid = tile_grid(n);
+  if (noise) {
+    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, true, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+    else hipLaunchKernelGGL((dropout_fwd_kernel<false, true, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+  } else {
+    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, false, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+    else hipLaunchKernelGGL((dropout_fwd_kernel<false, false, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+  }
+  return launch_status();
+}
 
 extern "C" {
 
@@ -288,25 +317,12 @@ int exact_leaky_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, f
 
 int exact_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p,
                           int64_t n, float* y, uint32_t* mask, void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
-  if (!(p >= 0.f && p < 1.f)) return EXACT_E_ARG;
-  if (n == 0) return EXACT_OK;
-  if (!x || !y || !mask) return EXACT_E_NULL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  // quantization_cuda_kernel.cu:456: float pinv = 1. / (1. - p), evaluated in double
-  const float pinv = static_cast<float>(1.0 / (1.0 - static_cast<double>(p)));
-  const uint32_t sl = static_cast<uint32_t>(seed), sh = static_cast<uint32_t>(seed >> 32);
-  const uint32_t ol = static_cast<uint32_t>(offset), oh = static_cast<uint32_t>(offset >> 32);
-  const bool v4 = aligned16(x) && aligned16(y) && (!noise || aligned16(noise));
-  const dim3 grid = tile_grid(n);
-  if (noise) {
-    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, true>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
-    else hipLaunchKernelGGL((dropout_fwd_kernel<false, true>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
-  } else {
-    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, false>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
-    else hipLaunchKernelGGL((dropout_fwd_kernel<false, false>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
-  }
-  return launch_status();
+  return dropout_forward<false>(x, noise, seed, offset, p, n, y, mask, stream);
+}
+
+int exact_relu_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p,
+                               int64_t n, float* y, uint32_t* mask, void* stream) {
+  return dropout_forward<true>(x, noise, seed, offset, p, n, y, mask, stream);
 }
 
 int exact_dropout_bwd_f32(const float* dy, const uint32_t* mask, float p, int64_t n, float* dx,

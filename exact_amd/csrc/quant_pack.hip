@@ -73,9 +73,23 @@ struct PackArgs {
   float* min_f32;
   uint16_t* scale_bf16;
   uint16_t* min_bf16;
+  // ACT form only: ReLU + dropout applied to x before the statistics
+  const float* act_noise;  // nullable
+  uint32_t act_seed_lo, act_seed_hi, act_off_lo, act_off_hi;
+  float p, pinv;
+  float* y;                // activation output [N, G]
+  uint8_t* mask_bytes;     // 1-bit mask of (x > 0) && keep, byte i / 8 holds elements i .. i + 7
+  int64_t mask_tail_begin, mask_tail_end;  // bytes of the last mask word no element maps to
 };
 
-template <int BITS, int OPT, int VEC, bool FULL, bool NOISE_IN, bool FUSED>
+// ACT: x first goes through ReLU and dropout (the arithmetic of
+// dropout_fwd_kernel<.., RELU = true>; noise from the flat Philox stream of the
+// mask kernels, block = flat index / 8), the result is written to y, its mask
+// bits to mask_bytes, and the row statistics / quantisation then work on that
+// result -- "ReLU -> dropout -> quantize_activation of the next layer's input"
+// in one pass.  Needs G % 8 == 0, so that an oct is one Philox block and one
+// mask byte.
+template <int BITS, int OPT, int VEC, bool FULL, bool NOISE_IN, bool FUSED, bool ACT = false>
 __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   constexpr int WPT = 8 / BITS;
   constexpr float B = static_cast<float>((1 << BITS) - 1);
@@ -103,6 +117,32 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       for (int i = 0; i < 8; ++i) v[k][i] = 0.f;
     } else {
       load_oct<VEC, FULL>(a.x + row_off + d0, nv[k], v[k]);
+    }
+    if constexpr (ACT) {
+      if (nv[k] > 0) {  // G % 8 == 0: a whole oct or nothing
+        const int64_t blk = (row_off + d0) >> 3;
+        float ud[8];
+        if constexpr (NOISE_IN) {
+          load_oct<VEC, true>(a.act_noise + row_off + d0, 8, ud);
+        } else {
+          const Philox4 r = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32),
+                                          a.act_off_lo, a.act_off_hi, a.act_seed_lo, a.act_seed_hi);
+          philox_uniform8(r, ud);
+        }
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const bool pos = v[k][i] > 0.f;
+          const bool keep = ud[i] > a.p;
+          float r = pos ? v[k][i] : 0.f;
+          r = r * (keep ? 1.f : 0.f);
+          r = r * a.pinv;
+          v[k][i] = r;
+          m |= static_cast<uint32_t>(pos && keep) << i;
+        }
+        store_oct<VEC, true>(a.y + row_off + d0, 8, v[k]);
+        a.mask_bytes[blk] = static_cast<uint8_t>(m);
+      }
     }
   }
 
@@ -203,7 +243,11 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       }
     }
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0 && t == 0) a.packed[a.pad_index] = 0;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && t == 0) {
+    a.packed[a.pad_index] = 0;
+    if constexpr (ACT)
+      for (int64_t i = a.mask_tail_begin; i < a.mask_tail_end; ++i) a.mask_bytes[i] = 0;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -350,7 +394,7 @@ static int pack_common(const float* x, const float* mn, const float* scale, cons
   }
 
   const Geometry g = plan_rows(G, do_fused ? 4 : 1);
-  PackArgs a;
+  PackArgs a{};
   a.x = x;
   a.noise = noise;
   a.mn_in = mn;
@@ -382,6 +426,32 @@ static int pack_common(const float* x, const float* mn, const float* scale, cons
     else launch_pack_bits<false, false>(a, bits, g.opt, vec4, full, grid, s);
   }
   return launch_status();
+}
+
+// ---- ReLU + dropout + statistics + pack (ACT form) ---------------------------
+template <int BITS, int OPT, bool NOISE_IN>
+static void launch_act_variant(const PackArgs& a, bool full, dim3 grid, hipStream_t s) {
+  if (full)
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, true, NOISE_IN, true, true>), grid, dim3(kBlock), 0, s, a);
+  else
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, false, NOISE_IN, true, true>), grid, dim3(kBlock), 0, s, a);
+}
+
+template <int BITS, bool NOISE_IN>
+static void launch_act_opt(const PackArgs& a, int opt, bool full, dim3 grid, hipStream_t s) {
+  if (opt == 4) return launch_act_variant<BITS, 4, NOISE_IN>(a, full, grid, s);
+  if (opt == 2) return launch_act_variant<BITS, 2, NOISE_IN>(a, full, grid, s);
+  launch_act_variant<BITS, 1, NOISE_IN>(a, full, grid, s);
+}
+
+template <bool NOISE_IN>
+static void launch_act_bits(const PackArgs& a, int bits, int opt, bool full, dim3 grid, hipStream_t s) {
+  switch (bits) {
+    case 1: return launch_act_opt<1, NOISE_IN>(a, opt, full, grid, s);
+    case 2: return launch_act_opt<2, NOISE_IN>(a, opt, full, grid, s);
+    case 4: return launch_act_opt<4, NOISE_IN>(a, opt, full, grid, s);
+    default: return launch_act_opt<8, NOISE_IN>(a, opt, full, grid, s);
+  }
 }
 
 }  // namespace exact
@@ -426,6 +496,65 @@ int exact_minmax_pack_f32(const float* x, const float* noise, uint64_t seed, uin
                           float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, void* stream) {
   return pack_common(x, nullptr, nullptr, noise, seed, offset, N, G, bits, packed, scale_f32, min_f32,
                      scale_bf16, min_bf16, true, static_cast<hipStream_t>(stream));
+}
+
+int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act_noise, uint64_t act_seed,
+                                       uint64_t act_offset, const float* noise, uint64_t seed, uint64_t offset,
+                                       int64_t N, int64_t G, int bits, float* y, uint32_t* mask, uint8_t* packed,
+                                       float* scale_f32, float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16,
+                                       void* stream) {
+  if (int rc = check_quant_shape(N, G, bits)) return rc;
+  if (!(p >= 0.f && p < 1.f)) return EXACT_E_ARG;
+  if ((act_noise == nullptr) != (noise == nullptr)) return EXACT_E_ARG;  // both streams supplied, or neither
+  if (G % 8 != 0 || G > 1024 || N * G > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+  if (!packed) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t pad_index = exact_packed_nbytes(N, G, bits) - 1;
+  if (N == 0 || G == 0) {
+    hipLaunchKernelGGL(zero_byte_kernel, dim3(1), dim3(1), 0, s, packed + pad_index);
+    return launch_status();
+  }
+  if (!x || !y || !mask) return EXACT_E_NULL;
+  if (!aligned(x, 16) || !aligned(y, 16) || (noise && (!aligned(noise, 16) || !aligned(act_noise, 16))))
+    return EXACT_E_ALIGN;
+  const Geometry g = plan_rows(G, 4);
+  PackArgs a{};
+  a.x = x;
+  a.noise = noise;
+  a.mn_in = nullptr;
+  a.scale_in = nullptr;
+  a.seed_lo = static_cast<uint32_t>(seed);
+  a.seed_hi = static_cast<uint32_t>(seed >> 32);
+  a.off_lo = static_cast<uint32_t>(offset);
+  a.off_hi = static_cast<uint32_t>(offset >> 32);
+  a.N = N;
+  a.G = static_cast<int>(G);
+  a.opr = g.opr;
+  a.lpr_log2 = g.lpr_log2;
+  a.packed = packed;
+  a.pad_index = pad_index;
+  a.scale_f32 = scale_f32;
+  a.min_f32 = min_f32;
+  a.scale_bf16 = scale_bf16;
+  a.min_bf16 = min_bf16;
+  a.out_vec = aligned(packed, 8) ? 8 : aligned(packed, 4) ? 4 : 1;
+  a.act_noise = act_noise;
+  a.act_seed_lo = static_cast<uint32_t>(act_seed);
+  a.act_seed_hi = static_cast<uint32_t>(act_seed >> 32);
+  a.act_off_lo = static_cast<uint32_t>(act_offset);
+  a.act_off_hi = static_cast<uint32_t>(act_offset >> 32);
+  a.p = p;
+  // quantization_cuda_kernel.cu:456: float pinv = 1. / (1. - p), evaluated in double
+  a.pinv = static_cast<float>(1.0 / (1.0 - static_cast<double>(p)));
+  a.y = y;
+  a.mask_bytes = reinterpret_cast<uint8_t*>(mask);
+  a.mask_tail_begin = N * G / 8;
+  a.mask_tail_end = (N * G + 31) / 32 * 4;
+  const int rows_per_wg = kBlock >> g.lpr_log2;
+  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), 1u);
+  if (noise) launch_act_bits<true>(a, bits, g.opt, g.full, grid, s);
+  else launch_act_bits<false>(a, bits, g.opt, g.full, grid, s);
+  return launch_status();
 }
 
 }  // extern "C"

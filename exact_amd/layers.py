@@ -9,7 +9,7 @@ from torch.nn import Parameter
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCNConv, SAGEConv, glorot
-from .ops import input2rp, qbatch_norm, qelu, qlinear, quantize_activation
+from .ops import input2rp, qbatch_norm, qelu, qlinear, quantize_activation, relu_dropout, take_compressed
 from .qsheme import QScheme
 from .spmm import QMatmul
 
@@ -22,6 +22,8 @@ class QLinear(torch.nn.Linear):
 
     def forward(self, input, quantized=None, randmat=None):  # noqa: A002
         if self.training:
+            if quantized is None:
+                quantized = take_compressed(input, project=self.rp)
             return qlinear.apply(input, self.weight, self.bias, quantized, randmat, self.scheme, self.rp)
         return super().forward(input)
 
@@ -49,7 +51,7 @@ class QGCNConv(GCNConv):
             # layers.py:252 passes lin_scheme in the `randmat` slot; with
             # kept_frac == 1 that slot is unused, so the numbers are those of
             # a qlinear without a scheme.  Here the scheme is passed as scheme.
-            x = qlinear.apply(x, self.weight, None, None, None, self.lin_scheme)
+            x = qlinear.apply(x, self.weight, None, take_compressed(x), None, self.lin_scheme)
         else:
             x = F.linear(x, self.weight, None)
         out = self.message_and_aggregate(adj_t, x)
@@ -90,7 +92,7 @@ class QSAGEConv(SAGEConv):
                 dim_reduced_input, randmat = input2rp(x[0], kept_acts)
             else:
                 dim_reduced_input, randmat = x[0], None
-            quantized = quantize_activation(dim_reduced_input, self.scheme)
+            quantized = take_compressed(x[0]) or quantize_activation(dim_reduced_input, self.scheme)
         else:
             quantized, randmat = None, None
         out = self.message_and_aggregate(edge_index, x, quantized=quantized, randmat=randmat)
@@ -160,6 +162,26 @@ class QDropout2(torch.nn.Module):
         if self.training:
             return ext_quantization.act_quantized_dropout(input, self.p, self.training) * (1 - self.p)
         return F.dropout(input, self.p, self.training) * (1 - self.p)
+
+
+class QReLUDropout(torch.nn.Module):
+    """QReLU followed by QDropout (layers.py:284-325) as one pass that keeps one
+    joint mask; with `for_consumer`, the compressed copy the following
+    QLinear / QGCNConv / QSAGEConv would make of the result is produced in the
+    same pass and handed to it.  Bit-identical to the separate layers."""
+
+    def __init__(self, p, for_consumer=True):
+        super().__init__()
+        self.p = p
+        self.for_consumer = for_consumer
+
+    def forward(self, input):  # noqa: A002
+        if self.training:
+            return relu_dropout(input, self.p, self.for_consumer)
+        return F.relu(input)
+
+    def extra_repr(self):
+        return f"p={self.p}, for_consumer={self.for_consumer}"
 
 
 class QBatchNorm1d(torch.nn.BatchNorm1d):

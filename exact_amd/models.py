@@ -5,7 +5,7 @@ them from stock layers (QModule then swaps the layers)."""
 import torch
 from torch.nn import BatchNorm1d, ModuleList
 
-from .nn import GCNConv, SAGEConv
+from .nn import GCNConv, ReLUDropout, SAGEConv
 
 
 class _Stack(torch.nn.Module):
@@ -13,11 +13,10 @@ class _Stack(torch.nn.Module):
                  dropout=0.0, batch_norm=False, residual=False, drop_input=False):
         super().__init__()
         self.in_channels, self.out_channels, self.num_layers = in_channels, out_channels, num_layers
-        self.dropout = torch.nn.Dropout(p=dropout)
+        self.act_drop = ReLUDropout(p=dropout)  # one module for the pair: QModule fuses it
         self.drop_input = drop_input
         if drop_input:
             self.input_dropout = torch.nn.Dropout(p=dropout)
-        self.activation = torch.nn.ReLU()
         self.batch_norm, self.residual = batch_norm, residual
         self.convs = ModuleList()
         for i in range(num_layers):
@@ -43,8 +42,7 @@ class _Stack(torch.nn.Module):
                 h = self.bns[idx](h)
             if self.residual and h.size(-1) == x.size(-1):
                 h = h + x[:h.size(0)]
-            x = self.activation(h)
-            x = self.dropout(x)
+            x = self.act_drop(h)
         return self.convs[-1](x, adj_t)
 
 

@@ -7,10 +7,10 @@ import torch
 import torch.nn as nn
 
 from .conf import config
-from .layers import QBatchNorm1d, QDropout, QDropout2, QGCNConv, QLinear, QReLU, QSAGEConv
-from .nn import GCNConv, SAGEConv
+from .layers import QBatchNorm1d, QDropout, QDropout2, QGCNConv, QLinear, QReLU, QReLUDropout, QSAGEConv
+from .nn import GCNConv, ReLUDropout, SAGEConv
 
-_QUANTIZED = (QBatchNorm1d, QLinear, QReLU, QGCNConv, QDropout, QDropout2, QSAGEConv)
+_QUANTIZED = (QBatchNorm1d, QLinear, QReLU, QGCNConv, QDropout, QDropout2, QSAGEConv, QReLUDropout)
 
 
 def _is_pyg(child, name):
@@ -37,6 +37,11 @@ class QModule(nn.Module):
                 new = QReLU()
             elif isinstance(child, nn.Dropout):
                 new = QDropout2(child.p) if config.dropout2 else QDropout(child.p)
+            elif isinstance(child, ReLUDropout):
+                if config.fuse_epilogue and not config.dropout2:
+                    new = QReLUDropout(child.p)
+                else:
+                    new = nn.Sequential(QReLU(), QDropout2(child.p) if config.dropout2 else QDropout(child.p))
             elif isinstance(child, GCNConv) or _is_pyg(child, "GCNConv"):
                 new = QGCNConv(child.in_channels, child.out_channels, child.improved, child.cached,
                                child.add_self_loops, child.normalize, child.bias is not None, aggr=child.aggr)

@@ -128,3 +128,18 @@ class SAGEConv(torch.nn.Module):
         if self.normalize:
             out = F.normalize(out, p=2.0, dim=-1)
         return out
+
+
+class ReLUDropout(torch.nn.Module):
+    """ReLU followed by dropout as ONE module, so that QModule can swap the
+    pair for a single fused pass (QReLUDropout)."""
+
+    def __init__(self, p=0.5):
+        super().__init__()
+        self.p = p
+
+    def forward(self, input):  # noqa: A002
+        return F.dropout(F.relu(input), self.p, self.training)
+
+    def extra_repr(self):
+        return f"p={self.p}"

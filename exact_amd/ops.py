@@ -18,6 +18,7 @@ import math
 import torch
 import torch.nn.functional as F
 from torch.autograd.function import Function
+from torch.utils.weak import WeakIdKeyDictionary
 
 from . import _lib
 from .conf import config
@@ -384,3 +385,72 @@ class qspmm_min(Function):
     @staticmethod
     def backward(ctx, grad_outputs):
         return _extreme_backward(ctx, grad_outputs)
+
+
+# ---------------------------------------------------------------------------
+# fused epilogue: ReLU -> dropout -> compressed copy for the consumer
+# ---------------------------------------------------------------------------
+class qrelu_dropout(Function):
+    """dropout(relu(input)) in one pass with one joint 1-bit mask kept for
+    backward -- the pair QReLU -> QDropout of the reference (layers.py:284-325).
+    With `bits`, the same pass also quantises the result the way the next
+    layer's quantize_activation would (ops.py:69-83) and returns that copy:
+    -> (output, packed | None, scale bf16 | None, min bf16 | None)."""
+
+    @staticmethod
+    def forward(ctx, input, p, bits=None):  # noqa: A002
+        flat = _rows_by_features(input) if input.dim() >= 2 else input
+        if bits is None:
+            out, mask = ext_quantization.relu_dropout_fwd(flat, p)
+            packed = scale = mn = None
+        else:
+            out, mask, packed, scale, mn = ext_quantization.relu_dropout_minmax_pack(flat, p, bits)
+            ctx.mark_non_differentiable(packed, scale, mn)
+        ctx.save_for_backward(mask)
+        ctx.p = float(p)
+        return out.view(input.shape), packed, scale, mn
+
+    @staticmethod
+    def backward(ctx, grad_output, *unused):
+        (mask,) = ctx.saved_tensors
+        return ext_quantization.dropout_bwd(grad_output, mask, ctx.p), None, None
+
+
+# Compressed copies made ahead of their consumer, keyed by the tensor they
+# describe.  The entry dies with the tensor; `_version` guards against an
+# in-place change between producer and consumer.
+_HANDED_OVER = WeakIdKeyDictionary()  # keyed by identity: Tensor.__eq__ is elementwise
+
+
+def hand_over_compressed(tensor, quantized):
+    _HANDED_OVER[tensor] = (tensor._version, quantized)
+
+
+def take_compressed(tensor, project=True):
+    """The compressed copy a fused producer made of exactly this tensor for a
+    consumer that would call quantize_activation(tensor) itself, or None."""
+    entry = _HANDED_OVER.pop(tensor, None) if isinstance(tensor, torch.Tensor) else None
+    if entry is None:
+        return None
+    version, quantized = entry
+    usable = (config.compress_activation and version == tensor._version
+              and quantized[1] == config.activation_compression_bits[0]
+              and not (project and config.kept_frac < 1.0))
+    return quantized if usable else None
+
+
+def relu_dropout(input, p, for_consumer=False):  # noqa: A002
+    """dropout(relu(input)); with `for_consumer`, the compressed copy of the
+    result is made in the same pass where the kernel can (2-D rows of a
+    multiple of 8 <= 1024 columns, compression on, no projection) and handed
+    over to the layer that receives the result."""
+    check_device_tensor(input, "input")
+    bits = None
+    if (for_consumer and config.compress_activation and config.kept_frac == 1.0 and input.dim() == 2
+            and ext_quantization.fusable_width(input.shape[1])):
+        _unsupported_modes()
+        bits = config.activation_compression_bits[0]
+    out, packed, scale, mn = qrelu_dropout.apply(input, p, bits)
+    if bits is not None:
+        hand_over_compressed(out, (packed, bits, scale, mn))
+    return out

@@ -150,6 +150,33 @@ int exact_leaky_relu_fwd_f32(const float *x, int64_t n, float slope, float *y,
 int exact_leaky_relu_bwd_f32(const float *dy, const uint32_t *mask, int64_t n,
                              float slope, float *dx, void *stream);
 
+/* Fused epilogues (no single counterpart in the reference: each replaces a
+ * chain of its calls with one pass over the data, bit-identical to the chain).
+ *
+ * ReLU then dropout: y = dropout(relu(x)) with ONE mask, bit = (x > 0) && keep;
+ * replaces act_quantized_relu followed by act_quantized_dropout
+ * (quantization.cc:66-84, 111-134).  The backward of the pair is
+ * exact_dropout_bwd_f32 on that mask.  Noise as in exact_dropout_fwd_f32. */
+int exact_relu_dropout_fwd_f32(const float *x, const float *noise, uint64_t seed,
+                               uint64_t offset, float p, int64_t n, float *y,
+                               uint32_t *mask, void *stream);
+
+/* ReLU, dropout and the quantisation of the result (the next layer's saved
+ * input) in one pass over x[N, G]: y and mask as exact_relu_dropout_fwd_f32
+ * with (act_noise | act_seed, act_offset); packed / scale / min as
+ * exact_minmax_pack_f32 applied to y with (noise | seed, offset).  Replaces
+ * layers.py:288-292 + :321-325 + the quantize_activation of the following
+ * qlinear (ops.py:149).  Needs G % 8 == 0, G <= 1024, 16-byte aligned x, y and
+ * noise (else EXACT_E_SHAPE / EXACT_E_ALIGN: call the separate entry points);
+ * act_noise and noise are both given or both NULL. */
+int exact_relu_dropout_minmax_pack_f32(const float *x, float p, const float *act_noise,
+                                       uint64_t act_seed, uint64_t act_offset,
+                                       const float *noise, uint64_t seed, uint64_t offset,
+                                       int64_t N, int64_t G, int bits, float *y,
+                                       uint32_t *mask, uint8_t *packed, float *scale_f32,
+                                       float *min_f32, uint16_t *scale_bf16,
+                                       uint16_t *min_bf16, void *stream);
+
 /* a7. Random projection: out[N, k] = X[N, D] . R[D, k]  (input2rp, ops.py:107-118)
  * and back: out[N, D] = Xr[N, k] . R[D, k]^T  (rp2input, ops.py:121-125).
  * fp32 in, fp32 accumulate on the matrix cores. */

@@ -254,6 +254,46 @@ static void check_leaky(int64_t n, std::mt19937& rng) {
   CHECK(bad == 0, "leaky relu differs n=%ld: %ld", (long)n, (long)bad);
 }
 
+// ReLU -> dropout (-> statistics + pack) in one pass against the chain of the
+// oracle's separate functions.
+static void check_fused(int64_t N, int64_t G, int bits, bool supplied, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 2.f);
+  std::uniform_real_distribution<float> ud(0.f, 1.f);
+  const int64_t n = N * G, words = (n + 31) / 32;
+  Buf<float> x(n), ua(n), uq(n), y1(n), y2(n), y(n), mn(N), mx(N), sc(N), mn2(N), sc2(N);
+  Buf<uint32_t> m1(words), m2(words), m(words);
+  for (int64_t i = 0; i < n; ++i) {
+    x[i] = nd(rng); ua[i] = ud(rng); uq[i] = ud(rng);
+    if (ua[i] >= 1.f) ua[i] = 0.5f;
+    if (uq[i] >= 1.f) uq[i] = 0.5f;
+  }
+  const float p = 0.4f;
+  const uint64_t s1 = 0x51ull, o1 = 8, s2 = 0x77ull, o2 = (3ull << 32) + 12;
+  oracle_relu_fwd(x.p, n, y1.p, m1.p);
+  oracle_dropout_fwd(y1.p, supplied ? ua.p : nullptr, s1, o1, p, n, y2.p, m2.p);
+  const int64_t nb = exact_packed_nbytes(N, G, bits);
+  Buf<uint8_t> packed(nb), want(nb);
+  Buf<uint16_t> sbf(N), mbf(N);
+  oracle_row_minmax(y2.p, N, G, mn.p, mx.p);
+  oracle_scale(mn.p, mx.p, N, bits, sc.p);
+  std::memset(want.p, 0, nb);
+  oracle_pack(y2.p, mn.p, sc.p, supplied ? uq.p : nullptr, s2, o2, N, G, bits, want.p);
+  int rc = exact_relu_dropout_fwd_f32(x.p, supplied ? ua.p : nullptr, s1, o1, p, n, y.p, m.p, nullptr);
+  int64_t bad = 0;
+  for (int64_t i = 0; i < words; ++i) bad += m[i] != (m1[i] & m2[i]);
+  CHECK(rc == 0 && std::memcmp(y.p, y2.p, n * 4) == 0 && bad == 0, "relu_dropout differs N=%ld G=%ld", (long)N, (long)G);
+  if (G % 8 != 0 || G > 1024) return;
+  std::memset(y.p, 0xFF, n * 4);
+  std::memset(m.p, 0xFF, words * 4);
+  rc = exact_relu_dropout_minmax_pack_f32(x.p, p, supplied ? ua.p : nullptr, s1, o1, supplied ? uq.p : nullptr, s2, o2,
+                                          N, G, bits, y.p, m.p, packed.p, sc2.p, mn2.p, sbf.p, mbf.p, nullptr);
+  bad = 0;
+  for (int64_t i = 0; i < words; ++i) bad += m[i] != (m1[i] & m2[i]);
+  CHECK(rc == 0 && std::memcmp(y.p, y2.p, n * 4) == 0 && bad == 0, "fused y/mask differ N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  CHECK(std::memcmp(packed.p, want.p, nb) == 0, "fused packed differs N=%ld G=%ld bits=%d supplied=%d", (long)N, (long)G, bits, supplied);
+  CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "fused scale/min differ N=%ld G=%ld", (long)N, (long)G);
+}
+
 int main(int argc, char** argv) {
   std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
@@ -287,6 +327,12 @@ int main(int argc, char** argv) {
   check_extra(40, 40, 1, 3, rng);
   check_extra(50, 50, 1000, 3, rng);
   std::printf("leaky / minmax / sddmm ok (failures so far %d)\n", g_fail);
+  const int64_t fs[][2] = {{1, 8}, {5, 16}, {37, 40}, {64, 256}, {203, 256}, {100, 128}, {33, 1024}, {19, 520},
+                           {129, 104}, {12, 768}, {7, 12}, {3, 1032}};
+  for (auto& f : fs)
+    for (int bits : {1, 2, 4, 8})
+      for (int supplied = 0; supplied < 2; ++supplied) check_fused(f[0], f[1], bits, supplied, rng);
+  std::printf("fused epilogues ok (failures so far %d)\n", g_fail);
   if (mode == "full") {
     for (int bits : {1, 2, 4, 8}) check_quant(169343, 256, bits, bits == 2, rng);
     std::printf("full-size quant ok (failures so far %d)\n", g_fail);
@@ -294,6 +340,7 @@ int main(int argc, char** argv) {
     check_spmm(169343, 169343, 256, 14, 20000, rng);
     check_spmm(169343, 169343, 40, 14, 20000, rng);
     check_rp(169343, 256, 32, rng);
+    check_fused(169343, 256, 2, false, rng);
     std::printf("full-size spmm/rp/masks ok (failures so far %d)\n", g_fail);
   }
   std::printf(g_fail ? "FAILED: %d check(s)\n" : "all checks passed\n", g_fail);

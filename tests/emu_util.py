@@ -209,3 +209,40 @@ def sddmm(row, rowptr, col, mat, grad, reduce, idx=np.int64, guard=8):
     assert rc == 0, rc
     assert (out[row.size:] == np.float32(-777.0)).all()
     return out[:row.size]
+
+
+def relu_dropout_fwd(x, prob, noise=None, seed=0, offset=0, guard=8):
+    x = f32(x).reshape(-1)
+    n = x.size
+    y = np.full(n + guard, np.float32(7.0), np.float32)
+    words = (n + 31) // 32
+    mask = np.full(words + guard, 0x5A5A5A5A, np.uint32)
+    noise = None if noise is None else f32(noise).reshape(-1)
+    assert emu().exact_relu_dropout_fwd_f32(p(x), p(noise), seed, offset, prob, n, p(y), p(mask), None) == 0
+    assert (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
+    return y[:n], mask[:words]
+
+
+def relu_dropout_minmax_pack(x, prob, bits, act_noise=None, noise=None, act_seed=0, act_offset=0, seed=0, offset=0,
+                             guard=64, expect_rc=0):
+    """-> (y, mask words, packed, scale f32, min f32, scale bf16 bits, min bf16 bits)."""
+    x = f32(x)
+    N, G = x.shape
+    n = N * G
+    nb = int(emu().exact_packed_nbytes(N, G, bits))
+    packed = np.full(nb + guard, 0xA5, np.uint8)
+    y = np.full(n + guard, np.float32(7.0), np.float32)
+    words = (n + 31) // 32
+    mask = np.full(words + guard, 0x5A5A5A5A, np.uint32)
+    s32, m32 = np.zeros(N, np.float32), np.zeros(N, np.float32)
+    sbf, mbf = np.zeros(N, np.uint16), np.zeros(N, np.uint16)
+    act_noise = None if act_noise is None else f32(act_noise)
+    noise = None if noise is None else f32(noise)
+    rc = emu().exact_relu_dropout_minmax_pack_f32(p(x), prob, p(act_noise), act_seed, act_offset, p(noise), seed,
+                                                  offset, N, G, bits, p(y), p(mask), p(packed), p(s32), p(m32), p(sbf),
+                                                  p(mbf), None)
+    assert rc == expect_rc, rc
+    if rc != 0:
+        return None
+    assert (packed[nb:] == 0xA5).all() and (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
+    return y[:n].reshape(N, G), mask[:words], packed[:nb], s32, m32, sbf, mbf

@@ -58,7 +58,7 @@ def test_harness_runs_every_part_at_tiny_scale(cpu_harness):
     logs = []
     out = bm.run(x, logs.append, scale=0.0005, epochs=1, warmup=0)
     assert "error" not in out["kernels"], out["kernels"]
-    for name in ("relu_fwd", "relu_bwd", "dropout_fwd", "dropout_bwd", "rp_fwd", "rp_bwd", "rp_compress_int2",
+    for name in ("relu_fwd", "relu_bwd", "dropout_fwd", "dropout_bwd", "relu_dropout_fwd", "rp_fwd", "rp_bwd", "rp_compress_int2",
                  "rp_decompress_int2"):
         assert out["kernels"][name]["us"] > 0
     for name in bm.EPOCH_CONFIGS:

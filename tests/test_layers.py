@@ -251,7 +251,11 @@ def test_qmodule_conversion_and_state_dict(backend):
     q = exact.QModule(net)
     kinds = [type(m).__name__ for m in q.model.modules()]
     assert kinds.count("QGCNConv") == 3 and kinds.count("QBatchNorm1d") == 2
-    assert "QReLU" in kinds and "QDropout" in kinds and "GCNConv" not in kinds
+    assert "QReLUDropout" in kinds and "QReLU" not in kinds and "GCNConv" not in kinds
+    config.fuse_epilogue = False
+    separate = [type(m).__name__ for m in exact.QModule(GCN(16, 32, 4, 3, dropout=0.3)).model.modules()]
+    assert "QReLU" in separate and "QDropout" in separate and "QReLUDropout" not in separate
+    config.fuse_epilogue = True
     assert [k for k in q.state_dict().keys()] == ref_keys       # the "model." prefix is stripped
     q.load_state_dict(q.state_dict())
     s = exact.QModule(SAGE(16, 32, 4, 2))

@@ -146,3 +146,202 @@ def test_edge_value_gradient(backend, reduce):
         got = value.grad.cpu().numpy()
         assert np.abs(got - want).max() <= tol * max(1.0, np.abs(want).max()), (compress, np.abs(got - want).max())
         assert x.grad is not None
+
+
+# ------------------------------------------------------------ fused epilogues (emulated kernels)
+def _chain(x, prob, bits, act_noise, noise):
+    """The chain the fused kernels replace, from the oracle's separate ops."""
+    N, G = x.shape
+    y1, m1 = o.relu_fwd(x.reshape(-1))
+    y2, m2 = o.dropout_fwd(y1, prob, act_noise.reshape(-1))
+    y2 = y2.reshape(N, G)
+    packed, _, sbf, mbf, scale, mn = o.quantize_activation(y2, bits, noise)
+    return y2, m1 & m2, packed, scale, mn, sbf, mbf
+
+
+@pytest.mark.parametrize("n", [1, 7, 33, 257, 2049, 10007])
+@pytest.mark.parametrize("supplied", [True, False])
+def test_relu_dropout_kernel_equals_the_two_kernels(n, supplied):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(F32)
+    noise = rng.random(n, dtype=F32) if supplied else o.philox_noise_flat(77, 5, n)
+    y, mask = e.relu_dropout_fwd(x, 0.4, noise if supplied else None, 77, 5)
+    y1, m1 = o.relu_fwd(x)
+    y2, m2 = o.dropout_fwd(y1, 0.4, noise)
+    assert np.array_equal(y.view(np.uint32), y2.view(np.uint32)) and np.array_equal(mask, m1 & m2)
+    # backward of the pair = dropout backward on the joint mask
+    g = rng.standard_normal(n).astype(F32)
+    want = o.relu_bwd(o.dropout_bwd(g, m2, 0.4), m1)
+    assert np.array_equal(e.dropout_bwd(g, mask, 0.4).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("N,G", [(1, 8), (5, 16), (37, 40), (64, 256), (203, 256), (100, 128), (33, 1024), (19, 520),
+                                 (129, 104), (12, 768)])
+@pytest.mark.parametrize("supplied", [True, False])
+def test_relu_dropout_pack_kernel_equals_the_chain(N, G, bits, supplied):
+    rng = np.random.default_rng(N * 1000 + G + bits)
+    x = (rng.standard_normal((N, G)) * 2).astype(F32)
+    if N > 3:
+        x[2] = -np.abs(x[2])                      # a row that ReLU zeroes entirely -> constant row
+    if supplied:
+        act_noise, noise = rng.random((N, G), dtype=F32), rng.random((N, G), dtype=F32)
+    else:
+        act_noise = o.philox_noise_flat(11, 3, N * G).reshape(N, G)
+        noise = o.philox_noise_rows(12, 4, N, G)
+    got = e.relu_dropout_minmax_pack(x, 0.5, bits, act_noise if supplied else None, noise if supplied else None,
+                                     11, 3, 12, 4)
+    want = _chain(x, 0.5, bits, act_noise, noise)
+    names = ("y", "mask", "packed", "scale", "min", "scale_bf16", "min_bf16")
+    for name, g_, w_ in zip(names, got, want):
+        g_, w_ = np.ascontiguousarray(g_), np.ascontiguousarray(w_)
+        assert g_.shape == w_.shape or g_.size == w_.size, name
+        assert g_.tobytes() == w_.tobytes(), name
+
+
+def test_relu_dropout_pack_kernel_rejects_what_it_cannot_do():
+    x = np.zeros((4, 12), F32)
+    assert e.relu_dropout_minmax_pack(x, 0.5, 2, expect_rc=-3) is None          # G % 8 != 0
+    assert e.relu_dropout_minmax_pack(np.zeros((2, 1032), F32), 0.5, 2, expect_rc=-3) is None
+    assert e.relu_dropout_minmax_pack(np.zeros((4, 16), F32), 1.0, 2, expect_rc=-5) is None
+    assert e.relu_dropout_minmax_pack(np.zeros((4, 16), F32), 0.5, 3, expect_rc=-2) is None
+    assert e.relu_dropout_minmax_pack(np.zeros((4, 16), F32), 0.5, 2, act_noise=np.zeros((4, 16), F32), expect_rc=-5) is None
+
+
+# ------------------------------------------------------------ fused epilogue (layers, both back ends)
+def _train_steps(backend, fuse, noise_seed, philox_seed, kept_frac=1.0, bits=2, steps=3, hidden=64):
+    """A few SGD steps of a 3-layer GCN; -> (losses, final weights)."""
+    from exact_amd.models import GCN
+    from exact_amd.sparse import gcn_norm
+    from gpu_util import SeededNoise
+    config.fuse_epilogue = fuse
+    config.kept_frac = kept_frac
+    config.activation_compression_bits = [bits]
+    if noise_seed is None:
+        config.noise_source = None
+        torch.manual_seed(philox_seed)
+        if backend.type == "cuda":
+            torch.cuda.manual_seed(philox_seed)
+    else:
+        s = SeededNoise(noise_seed)
+        config.noise_source, config.rp_matrix_source = s.noise_source, s.rp_matrix_source
+    A = csr(300, 300, 2400, 9, empty_rows=False)
+    adj = gcn_norm(SparseTensor.from_scipy(A).set_value(None), add_self_loops=True).to(backend)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(300, 48, generator=g).to(backend)
+    labels = torch.randint(0, 5, (300,), generator=g).to(backend)
+    torch.manual_seed(11)
+    net = GCN(48, hidden, 5, 3, dropout=0.5, batch_norm=True)
+    model = exact.QModule(net).to(backend).train()
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    losses = []
+    for _ in range(steps):
+        opt.zero_grad()
+        loss = F.cross_entropy(model(x, adj), labels)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    return losses, [p.detach().cpu().clone() for p in model.parameters()]
+
+
+def _same_training(backend, l_a, w_a, l_b, w_b):
+    if backend.type == "cpu":
+        assert l_a == l_b and all(torch.equal(a, b) for a, b in zip(w_a, w_b))
+    else:
+        # the GPU SpMM adds the partial sums of split rows with fp32 atomics, in no fixed
+        # order, so two runs of the SAME configuration already differ in the last bits
+        assert np.allclose(l_a, l_b, rtol=0, atol=1e-3)
+        assert all(torch.allclose(a, b, rtol=1e-3, atol=1e-3) for a, b in zip(w_a, w_b))
+
+
+@pytest.mark.parametrize("kept_frac,bits", [(1.0, 2), (1.0, 8), (0.25, 1)])
+def test_fused_epilogue_is_bit_identical_to_separate_layers(backend, kept_frac, bits):
+    """Same supplied noise in the same order: the fused ReLU -> dropout ->
+    quantise pass and the three separate layers give identical training."""
+    l_sep, w_sep = _train_steps(backend, False, 5, 0, kept_frac, bits)
+    l_fus, w_fus = _train_steps(backend, True, 5, 0, kept_frac, bits)
+    _same_training(backend, l_sep, w_sep, l_fus, w_fus)
+
+
+def test_fused_epilogue_uses_the_handed_over_copy(backend, monkeypatch):
+    """kept_frac 1: the consumer adopts the copy made by the fused pass (no
+    second quantisation of that tensor); an in-place change voids it."""
+    from exact_amd import ops
+    config.noise_source = None
+    x = torch.randn(64, 32, device=backend)
+    layer = exact.QReLUDropout(0.5).train()
+    y = layer(x)
+    q = ops.take_compressed(y)
+    assert q is not None and q[1] == 2 and ops.take_compressed(y) is None       # taken once
+    restored = ops.dequantize_activation(q, y.shape)
+    scale = q[2].float()
+    assert ((restored - y).abs() <= (1.0 / scale + 0.01 * y.abs().amax(1)).unsqueeze(1) + 1e-6)[torch.isfinite(scale)].all()
+    y2 = layer(x)
+    y2.mul_(2.0)
+    assert ops.take_compressed(y2) is None                                      # stale after an in-place op
+    y3 = layer(x)
+    config.activation_compression_bits = [4]
+    assert ops.take_compressed(y3) is None                                      # made for another bit width
+    config.activation_compression_bits = [2]
+    # widths the fused kernel does not take fall back to the mask-only pass
+    y4 = layer(torch.randn(10, 12, device=backend))
+    assert ops.take_compressed(y4) is None
+    # gradient of the pair
+    xg = torch.randn(50, 40, device=backend, requires_grad=True)
+    yg = layer(xg)
+    yg.backward(torch.ones_like(yg))
+    assert torch.equal(xg.grad, (yg.detach() != 0).float() * 2.0)
+    calls = []
+    real = ops.quantize_activation
+    monkeypatch.setattr(ops, "quantize_activation", lambda *a, **k: calls.append(1) or real(*a, **k))
+    lin = exact.QLinear(40, 8).to(backend).train()
+    lin(layer(xg.detach())).sum().backward()
+    assert calls == []                                                          # adopted, not re-quantised
+    lin(xg.detach()).sum().backward()
+    assert calls == [1]
+
+
+def test_fused_epilogue_with_internal_philox_noise(backend, monkeypatch):
+    """Internal noise: the fused pass draws (dropout, quantiser) in the order
+    the separate layers do, so a seeded run is again identical."""
+    import itertools
+
+    def reseed():
+        if backend.type == "cpu":   # the emulated back end numbers its draws itself: restart the numbering
+            counter = itertools.count(1)
+            monkeypatch.setattr(extq, "next_philox", lambda device: (0xC0FFEE, 4 * next(counter)))
+
+    reseed()
+    l_sep, w_sep = _train_steps(backend, False, None, 123)
+    reseed()
+    l_fus, w_fus = _train_steps(backend, True, None, 123)
+    _same_training(backend, l_sep, w_sep, l_fus, w_fus)
+
+
+@pytest.mark.parametrize("supplied", [True, False])
+@pytest.mark.parametrize("N,G,bits", [(203, 256, 2), (64, 128, 1), (37, 40, 4), (33, 1024, 8), (1000, 64, 2)])
+def test_fused_shims_match_the_oracle_chain(backend, monkeypatch, N, G, bits, supplied):
+    """The two fused entry points through the Python shims, on both back ends,
+    against relu -> dropout -> quantize_activation of the oracle (bytes)."""
+    from gpu_util import FixedNoise, bytes_equal
+    rng = np.random.default_rng(N + G + bits)
+    x = (rng.standard_normal((N, G)) * 2).astype(F32)
+    x[1] = -np.abs(x[1])
+    if supplied:
+        act_noise, noise = rng.random((N, G), dtype=F32), rng.random((N, G), dtype=F32)
+        config.noise_source = FixedNoise([torch.from_numpy(act_noise), torch.from_numpy(noise), torch.from_numpy(act_noise)])
+    else:
+        draws = iter([(0xABCDEF12345, 8), (0xABCDEF12345, 12), (0xABCDEF12345, 8)])
+        monkeypatch.setattr(extq, "next_philox", lambda device: next(draws))
+        act_noise = o.philox_noise_flat(0xABCDEF12345, 8, N * G).reshape(N, G)
+        noise = o.philox_noise_rows(0xABCDEF12345, 12, N, G)
+    want = _chain(x, 0.3, bits, act_noise, noise)
+    xt = torch.from_numpy(x).to(backend)
+    y, mask, packed, sbf, mbf = extq.relu_dropout_minmax_pack(xt, 0.3, bits)
+    assert bytes_equal(y, want[0]) and bytes_equal(mask, want[1]) and bytes_equal(packed, want[2])
+    assert bytes_equal(sbf, want[5]) and bytes_equal(mbf, want[6])
+    y2, mask2 = extq.relu_dropout_fwd(xt, 0.3)
+    assert bytes_equal(y2, want[0]) and bytes_equal(mask2, want[1])
+    g = torch.from_numpy(rng.standard_normal((N, G)).astype(F32)).to(backend)
+    want_dx = o.dropout_bwd(g.cpu().numpy().reshape(-1), want[1], 0.3)
+    assert bytes_equal(extq.dropout_bwd(g, mask, 0.3), want_dx)
