@@ -8,10 +8,10 @@ from torch.nn import Parameter
 
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
-from .nn import GCNConv, SAGEConv, glorot
+from .nn import GCN2Conv, GCNConv, GraphConv, SAGEConv, glorot
 from .ops import input2rp, qbatch_norm, qelu, qlinear, quantize_activation, relu_dropout, take_compressed
 from .qsheme import QScheme
-from .spmm import QMatmul
+from .spmm import QMatmul, qmatmul
 
 
 class QLinear(torch.nn.Linear):
@@ -106,6 +106,59 @@ class QSAGEConv(SAGEConv):
 
     def message_and_aggregate(self, adj_t, x, quantized=None, randmat=None):
         return self.msg_and_aggr_func(adj_t, x[0], quantized=quantized, randmat=randmat)
+
+
+class QGraphConv(GraphConv):
+    """layers.py:181-212: both linear maps are QLinear, the aggregation a
+    quantised SpMM."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        in_channels = self.in_channels
+        if isinstance(in_channels, int):
+            in_channels = (in_channels, in_channels)
+        bias = self.lin_l.bias is not None
+        self.lin_l = QLinear(in_channels[0], self.out_channels, bias=bias, rp=True)
+        self.lin_r = QLinear(in_channels[1], self.out_channels, bias=False, rp=True)
+        self.msg_and_aggr_func = QMatmul(self.aggr)
+        self.reset_parameters()
+
+    def message_and_aggregate(self, adj_t, x):
+        return self.msg_and_aggr_func(adj_t, x[0])
+
+
+def qaddmm(input, mat1, mat2, beta=1.0, alpha=1):  # noqa: A002
+    """layers.py:27-28.  As there, the product is qlinear(mat1, mat2) = mat1 @
+    mat2^T (not torch.addmm's mat1 @ mat2): QGCN2Conv multiplies by the
+    transposed weight in the reference, and so does this."""
+    return beta * input + alpha * qlinear.apply(mat1, mat2, None)
+
+
+class QGCN2Conv(GCN2Conv):
+    """layers.py:66-120."""
+
+    def message_and_aggregate(self, adj_t, x):
+        return qmatmul(adj_t, x, reduce=self.aggr)
+
+    def _addmm(self, inp, mat, weight):
+        return qaddmm(inp, mat, weight, beta=1.0 - self.beta, alpha=self.beta)
+
+
+class QMLP(torch.nn.Sequential):
+    """layers.py:32-47: QLinear (-> QBatchNorm1d) -> QReLU -> QDropout blocks."""
+
+    def __init__(self, channels, norm, bias=True, dropout=0.0):
+        blocks = []
+        for i in range(1, len(channels)):
+            blocks.append(QLinear(channels[i - 1], channels[i], bias))
+            if i < len(channels) - 1:
+                if norm == "batch":
+                    blocks.append(QBatchNorm1d(channels[i], affine=True))
+                elif norm:
+                    raise NotImplementedError(f'Normalization layer "{norm}" not supported.')
+                blocks.append(QReLU())
+                blocks.append(QDropout(dropout))
+        super().__init__(*blocks)
 
 
 class QReLU(torch.nn.Module):

@@ -1,16 +1,20 @@
 """QModule: wrap a model and swap its stock layers for the quantised ones, as
 exact/exact/module.py:18-112 of the reference does for the layer types on this
-library's path (Linear, BatchNorm1d, ReLU, Dropout, GCNConv, SAGEConv)."""
+library's path (Linear, BatchNorm1d, ReLU, Dropout, GCNConv, SAGEConv, GCN2Conv,
+GraphConv, CustomGATConv; GENConv is not provided)."""
 from collections import OrderedDict
 
 import torch
 import torch.nn as nn
 
 from .conf import config
-from .layers import QBatchNorm1d, QDropout, QDropout2, QGCNConv, QLinear, QReLU, QReLUDropout, QSAGEConv
-from .nn import GCNConv, ReLUDropout, SAGEConv
+from .gatconv import QCustomGATConv
+from .layers import (QBatchNorm1d, QDropout, QDropout2, QGCN2Conv, QGCNConv, QGraphConv, QLinear, QReLU,
+                     QReLUDropout, QSAGEConv)
+from .nn import CustomGATConv, GCN2Conv, GCNConv, GraphConv, ReLUDropout, SAGEConv
 
-_QUANTIZED = (QBatchNorm1d, QLinear, QReLU, QGCNConv, QDropout, QDropout2, QSAGEConv, QReLUDropout)
+_QUANTIZED = (QBatchNorm1d, QLinear, QReLU, QGCNConv, QDropout, QDropout2, QSAGEConv, QReLUDropout, QGCN2Conv,
+              QGraphConv, QCustomGATConv)
 
 
 def _is_pyg(child, name):
@@ -48,6 +52,17 @@ class QModule(nn.Module):
             elif isinstance(child, SAGEConv) or _is_pyg(child, "SAGEConv"):
                 new = QSAGEConv(child.in_channels, child.out_channels, child.normalize, child.root_weight,
                                 child.lin_l.bias is not None)
+            elif isinstance(child, GCN2Conv):
+                new = QGCN2Conv(child.channels, alpha=child.alpha, theta=None, layer=None,
+                                shared_weights=child.weight2 is None, cached=child.cached,
+                                add_self_loops=child.add_self_loops, normalize=child.normalize)
+                new.beta = child.beta
+            elif isinstance(child, GraphConv):
+                new = QGraphConv(child.in_channels, child.out_channels, child.aggr, child.lin_l.bias is not None)
+            elif isinstance(child, CustomGATConv):
+                new = QCustomGATConv(child.in_channels, child.out_channels, child.heads, child.concat,
+                                     child.negative_slope, child.dropout, child.add_self_loops,
+                                     child.bias is not None, child.residual, child.use_attn_dst)
             else:
                 QModule.convert_layers(child)
                 continue

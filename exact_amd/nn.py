@@ -143,3 +143,188 @@ class ReLUDropout(torch.nn.Module):
 
     def extra_repr(self):
         return f"p={self.p}"
+
+
+class GraphConv(torch.nn.Module):
+    """out = lin_l(aggr_j w_ij x_j) + lin_r(x_i), the operator the reference's
+    QGraphConv subclasses (layers.py:181-212; torch_geometric 1.7 parameter
+    names lin_l / lin_r).  Edge weights are the values of the SparseTensor."""
+
+    def __init__(self, in_channels, out_channels, aggr="add", bias=True):
+        super().__init__()
+        self.in_channels, self.out_channels, self.aggr = in_channels, out_channels, aggr
+        if isinstance(in_channels, int):
+            in_channels = (in_channels, in_channels)
+        self.lin_l = Linear(in_channels[0], out_channels, bias=bias)
+        self.lin_r = Linear(in_channels[1], out_channels, bias=False)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.lin_l.reset_parameters()
+        self.lin_r.reset_parameters()
+
+    def message_and_aggregate(self, adj_t, x):
+        return matmul(adj_t, x[0], reduce=self.aggr)
+
+    def forward(self, x, edge_index, edge_weight=None, size=None):
+        if isinstance(x, torch.Tensor):
+            x = (x, x)
+        out = self.lin_l(self.message_and_aggregate(edge_index, x))
+        if x[1] is not None:
+            out = out + self.lin_r(x[1])
+        return out
+
+
+class GCN2Conv(torch.nn.Module):
+    """GCNII layer: out = (1 - beta) h + beta h W1 with h = (1 - alpha) A x +
+    alpha x_0 (shared weights), or the two-weight form; beta = log(theta /
+    layer + 1).  The operator the reference's QGCN2Conv subclasses
+    (layers.py:66-120)."""
+
+    def __init__(self, channels, alpha, theta=None, layer=None, shared_weights=True, cached=False,
+                 add_self_loops=True, normalize=True, aggr="add"):
+        super().__init__()
+        self.channels, self.alpha, self.aggr = channels, alpha, aggr
+        self.beta = 1.0 if theta is None or layer is None else math.log(theta / layer + 1)
+        self.cached, self.normalize, self.add_self_loops = cached, normalize, add_self_loops
+        self._cached_adj_t = None
+        self.weight1 = Parameter(torch.Tensor(channels, channels))
+        if shared_weights:
+            self.register_parameter("weight2", None)
+        else:
+            self.weight2 = Parameter(torch.Tensor(channels, channels))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        glorot(self.weight1)
+        glorot(self.weight2)
+        self._cached_adj_t = None
+
+    def _normalized(self, adj_t):
+        if not self.normalize:
+            return adj_t
+        if self._cached_adj_t is not None:
+            return self._cached_adj_t
+        out = gcn_norm(adj_t, self.add_self_loops)
+        if self.cached:
+            self._cached_adj_t = out
+        return out
+
+    def message_and_aggregate(self, adj_t, x):
+        return matmul(adj_t, x, reduce=self.aggr)
+
+    def _addmm(self, inp, mat, weight):
+        return (1.0 - self.beta) * inp + self.beta * (mat @ weight)
+
+    def forward(self, x, x_0, edge_index, edge_weight=None):
+        x = self.message_and_aggregate(self._normalized(edge_index), x) * (1 - self.alpha)
+        x_0 = self.alpha * x_0[:x.size(0)]
+        if self.weight2 is None:
+            out = x + x_0
+            return self._addmm(out, out, self.weight1)
+        return self._addmm(x, x, self.weight1) + self._addmm(x_0, x_0, self.weight2)
+
+
+def edge_softmax(score, row, num_rows):
+    """Softmax of score[E, H] over the entries that share a row (PyG's
+    utils.softmax: shift by the group maximum, + 1e-16 in the denominator)."""
+    idx = row.view(-1, 1).expand_as(score)
+    top = torch.full((num_rows, score.size(1)), float("-inf"), dtype=score.dtype, device=score.device)
+    top = top.scatter_reduce(0, idx, score.detach(), "amax", include_self=True)
+    e = (score - top.index_select(0, row)).exp()
+    denom = torch.zeros((num_rows, score.size(1)), dtype=score.dtype, device=score.device).index_add_(0, row, e)
+    return e / (denom.index_select(0, row) + 1e-16)
+
+
+class CustomGATConv(torch.nn.Module):
+    """Multi-head graph attention with an optional residual projection and an
+    optional separate destination attention vector -- the reference's
+    CustomGATConv (gatconv.py:18-144), on the SparseTensor path: entry (i, j)
+    of adj_t carries the message from j to i."""
+
+    def __init__(self, in_channels, out_channels, heads=1, concat=True, negative_slope=0.2, dropout=0.0,
+                 add_self_loops=True, bias=True, residual=True, use_attn_dst=True):
+        super().__init__()
+        self.in_channels, self.out_channels, self.heads, self.concat = in_channels, out_channels, heads, concat
+        self.negative_slope, self.dropout, self.add_self_loops = negative_slope, dropout, add_self_loops
+        self.residual, self.use_attn_dst = residual, use_attn_dst
+        self._build_linears(Linear)
+        self.att_l = Parameter(torch.Tensor(1, heads, out_channels))
+        self.att_r = Parameter(torch.Tensor(1, heads, out_channels)) if use_attn_dst else self.att_l
+        if bias:
+            self.bias = Parameter(torch.Tensor(heads * out_channels if concat else out_channels))
+        else:
+            self.register_parameter("bias", None)
+        self.reset_parameters()
+
+    def _build_linears(self, linear_cls):
+        width = self.heads * self.out_channels
+        if isinstance(self.in_channels, int):
+            self.lin_l = linear_cls(self.in_channels, width, bias=False)
+            self.lin_r = self.lin_l
+        else:
+            self.lin_l = linear_cls(self.in_channels[0], width, bias=False)
+            self.lin_r = linear_cls(self.in_channels[1], width, bias=False)
+        if self.residual:
+            self.res_fc = Linear(self.in_channels, width, bias=False)
+        else:
+            self.res_fc = None
+
+    def reset_parameters(self):
+        gain = torch.nn.init.calculate_gain("relu")
+        torch.nn.init.xavier_normal_(self.lin_l.weight, gain=gain)
+        torch.nn.init.xavier_normal_(self.lin_r.weight, gain=gain)
+        if self.res_fc is not None:
+            torch.nn.init.xavier_normal_(self.res_fc.weight, gain=gain)
+        torch.nn.init.xavier_normal_(self.att_l, gain=gain)
+        if self.use_attn_dst:
+            torch.nn.init.xavier_normal_(self.att_r, gain=gain)
+        if self.bias is not None:
+            self.bias.data.zero_()
+
+    def _edges(self, adj_t):
+        """(row, col, number of rows) of the graph with self loops set; kept for
+        the graph object last seen, since building it sorts the entries."""
+        cached = getattr(self, "_edge_cache", None)
+        if cached is None or cached[0] is not adj_t:
+            g = adj_t.fill_diag(1.0) if self.add_self_loops else adj_t
+            row, col, _ = g.coo()
+            cached = (adj_t, row.long(), col.long(), g.sparse_size(0))
+            self._edge_cache = cached
+        return cached[1], cached[2], cached[3]
+
+    # the two hooks the quantised subclass replaces
+    def _leaky_relu(self, score):
+        return F.leaky_relu(score, self.negative_slope)
+
+    def _attention_dropout(self, alpha):
+        return F.dropout(alpha, p=self.dropout, training=self.training)
+
+    def forward(self, x, edge_index, size=None):
+        H, C = self.heads, self.out_channels
+        if isinstance(x, torch.Tensor):
+            x_l = x_r = self.lin_l(x).view(-1, H, C)
+            alpha_l = (x_l * self.att_l).sum(dim=-1)
+            alpha_r = (x_r * self.att_r).sum(dim=-1) if self.use_attn_dst else alpha_l
+            x_res = x
+        else:
+            x_l = self.lin_l(x[0]).view(-1, H, C)
+            alpha_l = (x_l * self.att_l).sum(dim=-1)
+            alpha_r = None
+            if x[1] is not None:
+                alpha_r = (self.lin_r(x[1]).view(-1, H, C) * self.att_r).sum(dim=-1)
+            x_res = x[1]
+        row, col, num_rows = self._edges(edge_index)
+        score = alpha_l.index_select(0, col)
+        if alpha_r is not None:
+            score = score + alpha_r.index_select(0, row)
+        alpha = edge_softmax(self._leaky_relu(score), row, num_rows)
+        alpha = self._attention_dropout(alpha)
+        msg = x_l.index_select(0, col) * alpha.unsqueeze(-1)
+        out = torch.zeros((num_rows, H, C), dtype=msg.dtype, device=msg.device).index_add_(0, row, msg)
+        out = out.view(-1, H * C) if self.concat else out.mean(dim=1)
+        if self.res_fc is not None:
+            out = out + self.res_fc(x_res)
+        if self.bias is not None:
+            out = out + self.bias
+        return out
