@@ -212,8 +212,8 @@ def train_epochs(model, x, adj, labels, train_idx, epochs, warmup, lr=0.01):
 EPOCH_CONFIGS = {
     # name: (model, N, raw directed edges, features, hidden, classes, layers, bits, kept_frac, batch_norm, dropout)
     "cfg3_gcn_int2": ("gcn", 169343, 1_160_000, 128, 256, 40, 3, 2, 1.0, True, 0.5),
-    "cfg4_sage_int2_rp0.125": ("sage", 232965, 11_600_000, 602, 256, 41, 2, 2, 0.125, False, 0.5),
-    "cfg5_sage_int1_rp0.25": ("sage", 2449029, 61_900_000, 100, 256, 47, 3, 1, 0.25, False, 0.5),
+    "cfg4_sage_int2_rp0.125": ("sage", 232965, 13_250_000, 602, 256, 41, 2, 2, 0.125, False, 0.5),
+    "cfg5_sage_int1_rp0.25": ("sage", 2449029, 65_700_000, 100, 256, 47, 3, 1, 0.25, False, 0.5),
 }
 
 
