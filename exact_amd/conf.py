@@ -17,7 +17,7 @@ _REFERENCE_FIELDS = {
     "single_precision": True,             # read at layer construction: attach QScheme objects
     "dropout2": False,                    # QModule uses QDropout2 instead of QDropout
     "empty_cache_threshold": None,
-    "swap": False,                        # not provided here (raises when set)
+    "swap": False,                        # keep the packed codes in pinned host memory between fwd and bwd
     "amp": False,
     "debug_memory_op_forward": False,
     "debug_memory_op_backward": False,

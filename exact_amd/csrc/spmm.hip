@@ -23,6 +23,7 @@ namespace exact {
 
 constexpr int kChunk = 64;  // entries per wavefront == lanes per wavefront
 constexpr int kGather = 8;  // X rows in flight per lane
+constexpr int kXcds = 8;    // accelerator complex dies of an MI355X, each with its own L2
 
 template <int VEC> struct Vec;
 template <> struct Vec<4> { using T = float4; };
@@ -83,17 +84,32 @@ __global__ __launch_bounds__(kBlock) void spmm_chunk_kernel(const I* __restrict_
                                                             float* __restrict__ out) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-  const int64_t e0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kChunk;
+  // Workgroups are handed to the 8 XCDs round-robin by index; give each XCD a
+  // contiguous range of chunks, so that neighbouring CSR rows (which in real
+  // graphs share neighbours) gather through the same L2.  gridDim.x is a
+  // multiple of kXcds; logical indices past the last chunk fall out below.
+  const int64_t per_xcd = gridDim.x / kXcds;
+  const int64_t wg = static_cast<int64_t>(blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+  const int64_t e0 = (wg * (kBlock / kWave) + wave) * kChunk;
   if (e0 >= nnz) return;
   const int cnt = static_cast<int>(nnz - e0 < kChunk ? nnz - e0 : kChunk);
   const int64_t kcol = (static_cast<int64_t>(blockIdx.y) * kWave + lane) * VEC;
   const bool kok = kcol < K;
 
-  // row that owns entry e0: the last r with rowptr[r] <= e0
+  // Row that owns entry e0: the last r with rowptr[r] <= e0.  A 64-ary search:
+  // every round the 64 lanes probe 64 evenly spaced positions of [lo, hi) at
+  // once and a ballot picks the sub-interval, so a graph of M rows costs
+  // ceil(log64 M) dependent loads (3 for 169k rows) instead of log2 M.
+  // Invariant: rowptr[lo] <= e0, and hi == M or rowptr[hi] > e0.
   int64_t lo = 0, hi = M;
   while (hi - lo > 1) {
-    const int64_t mid = (lo + hi) >> 1;
-    if (static_cast<int64_t>(rowptr[mid]) <= e0) lo = mid; else hi = mid;
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t pos = lo + step * lane;
+    const bool le = pos < hi && static_cast<int64_t>(rowptr[pos]) <= e0;
+    const uint64_t hits = __ballot(le);                 // rowptr is sorted: a run of ones from lane 0
+    const int last = 63 - __builtin_clzll(hits | 1u);  // bit 0 is set by the invariant
+    lo += step * last;
+    hi = (lo + step < hi) ? lo + step : hi;
   }
   int64_t r = lo;
 
@@ -179,7 +195,8 @@ template <typename I, int VEC>
 static void spmm_dispatch(const I* rowptr, const I* col, const float* val, const float* X, int64_t M,
                           int64_t nnz, int64_t K, int reduce, float* out, hipStream_t s) {
   const int64_t chunks = (nnz + kChunk - 1) / kChunk;
-  const dim3 grid(static_cast<unsigned>((chunks + 3) / 4),
+  const int64_t wgs = (chunks + 3) / 4;
+  const dim3 grid(static_cast<unsigned>((wgs + kXcds - 1) / kXcds * kXcds),
                   static_cast<unsigned>((K + kWave * VEC - 1) / (kWave * VEC)));
   const dim3 block(kBlock);
   const bool mean = reduce == EXACT_REDUCE_MEAN;

@@ -27,16 +27,13 @@ from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import quantization as ext_quantization
 from .cpp_extension import spmm
 from .cpp_extension._checks import check_device_tensor, ptr
-from .utils import empty_cache
+from .utils import empty_cache, swap_to_cpu
 
 
 def _unsupported_modes():
     if config.simulate:
         raise NotImplementedError("config.simulate (torch fake-quantisation, reference ops.py:21-34) is not "
                                   "provided: this package only runs the packed kernels")
-    if config.swap:
-        raise NotImplementedError("config.swap (host offload of packed activations) is not provided: "
-                                  "compressed activations stay resident in HBM")
 
 
 def _rows_by_features(t):
@@ -62,6 +59,8 @@ def quantize_and_pack(data, bits, mn, mx):
         raise TypeError("bits must be an int")
     scale = (2 ** bits - 1) / (mx - mn)      # reciprocal() * int, as torch evaluates it
     packed = ext_quantization.pack_single_precision(data, mn, mx, scale.to(data.dtype), bits, config.stochastic)
+    if config.swap:
+        packed = swap_to_cpu(packed)         # reference ops.py:41-42
     return packed, scale
 
 
@@ -70,6 +69,8 @@ def dequantize_and_unpack(data, shape, bits, scale, mn):
     quantize_activation returned."""
     _unsupported_modes()
     rows, feats = shape[0], math.prod(shape[1:])
+    if data.device != scale.device:          # offloaded by config.swap (reference ops.py:50-51)
+        data = data.to(scale.device, non_blocking=True)
     unpack = ext_quantization.unpack_bf16param if scale.dtype == torch.bfloat16 else ext_quantization.unpack_single_precision
     return unpack(data, bits, scale, mn, rows, feats)
 
@@ -86,6 +87,8 @@ def quantize_activation(input, scheme):  # noqa: A002
     check_device_tensor(input, "input")
     bits = config.activation_compression_bits[0]
     packed, scale_bf16, min_bf16 = ext_quantization.minmax_pack(_rows_by_features(input), bits)
+    if config.swap:
+        packed = swap_to_cpu(packed)
     return packed, bits, scale_bf16, min_bf16
 
 
@@ -452,5 +455,5 @@ def relu_dropout(input, p, for_consumer=False):  # noqa: A002
         bits = config.activation_compression_bits[0]
     out, packed, scale, mn = qrelu_dropout.apply(input, p, bits)
     if bits is not None:
-        hand_over_compressed(out, (packed, bits, scale, mn))
+        hand_over_compressed(out, (swap_to_cpu(packed) if config.swap else packed, bits, scale, mn))
     return out

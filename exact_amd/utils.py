@@ -27,6 +27,15 @@ def cast_adj(data):
         setattr(storage, field, cast_low_bit_int(getattr(storage, field)))
 
 
+def swap_to_cpu(tensor):
+    """Asynchronous copy of a device tensor into pinned host memory on the
+    current stream (reference utils.py:31-34).  The copy back
+    (`.to(device, non_blocking=True)` on the same stream) is ordered after it."""
+    host = torch.empty(tensor.shape, dtype=tensor.dtype, device="cpu", pin_memory=tensor.is_cuda)
+    host.copy_(tensor, non_blocking=True)
+    return host
+
+
 def get_memory_usage(gpu, print_info=False):
     """Bytes currently allocated by torch on device `gpu`."""
     allocated = torch.cuda.memory_allocated(gpu)

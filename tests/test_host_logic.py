@@ -43,10 +43,7 @@ def test_unsupported_modes_raise_instead_of_falling_back():
     config.simulate = True
     with pytest.raises(NotImplementedError, match="simulate"):
         ops.quantize_activation(x, None)
-    config.simulate, config.swap = False, True
-    with pytest.raises(NotImplementedError, match="swap"):
-        ops.quantize_activation(x, None)
-    config.swap, config.compress_activation = False, False
+    config.simulate, config.compress_activation = False, False
     assert ops.quantize_activation(x, None) == (x, None, None, None)
     assert ops.dequantize_activation((x, None, None, None), x.shape) is x
 

@@ -345,3 +345,29 @@ def test_fused_shims_match_the_oracle_chain(backend, monkeypatch, N, G, bits, su
     g = torch.from_numpy(rng.standard_normal((N, G)).astype(F32)).to(backend)
     want_dx = o.dropout_bwd(g.cpu().numpy().reshape(-1), want[1], 0.3)
     assert bytes_equal(extq.dropout_bwd(g, mask, 0.3), want_dx)
+
+
+def test_swap_keeps_the_packed_codes_on_the_host(backend):
+    """config.swap (reference ops.py:41-42, 50-51): between forward and backward
+    the packed codes live in (pinned) host memory; results do not change."""
+    from exact_amd import ops
+    from gpu_util import SeededNoise
+    x = torch.randn(200, 64, device=backend)
+    outs = []
+    for swap in (False, True):
+        config.swap = swap
+        s = SeededNoise(3)
+        config.noise_source = s.noise_source
+        q = ops.quantize_activation(x, None)
+        assert q[0].device.type == "cpu" if swap else q[0].device == x.device
+        if swap and backend.type == "cuda":
+            assert q[0].is_pinned()
+        outs.append((q[0].cpu().clone(), ops.dequantize_activation(q, x.shape)))
+        lin = exact.QLinear(64, 16).to(backend).train()
+        y = lin(exact.QReLUDropout(0.5).train()(x))       # the handed-over copy is offloaded too
+        y.sum().backward()
+        assert torch.isfinite(lin.weight.grad).all()
+        mn, mx = x.min(1).values, x.max(1).values
+        packed2, _ = ops.quantize_and_pack(x, 2, mn, mx)
+        assert (packed2.device.type == "cpu") == (swap or backend.type == "cpu")
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
