@@ -31,6 +31,11 @@ inline int launch_status() {
 // Block function of Salmon et al. (SC'11); the reference draws from cuRAND's
 // Philox4_32_10 (quantization_cuda_kernel.cu:77-79, 452-453).  The key is
 // wave-uniform, so its schedule lives in scalar registers.
+// a ^ b ^ c in one instruction (v_bitop3_b32, truth table 0x96 = odd parity)
+__device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
+  return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+}
+
 struct Philox4 {
   uint32_t x, y, z, w;
 };
@@ -43,8 +48,8 @@ __device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
   for (int r = 0; r < 10; ++r) {
     const uint64_t p0 = static_cast<uint64_t>(M0) * c0;
     const uint64_t p1 = static_cast<uint64_t>(M1) * c2;
-    const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0;
-    const uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n0 = xor3(static_cast<uint32_t>(p1 >> 32), c1, k0);
+    const uint32_t n2 = xor3(static_cast<uint32_t>(p0 >> 32), c3, k1);
     c1 = static_cast<uint32_t>(p1);
     c3 = static_cast<uint32_t>(p0);
     c0 = n0;
@@ -77,10 +82,10 @@ __device__ __forceinline__ void philox_uniform8(const Philox4& r, float (&u)[8])
 // fp32 -> bf16 bits, round to nearest even (what Tensor.to(torch.bfloat16)
 // does at ops.py:80-81 of the reference).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-  uint32_t b = __float_as_uint(f);
-  if ((b & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((b >> 16) & 0x8000u) | 0x7FC0u;
-  b += 0x7FFFu + ((b >> 16) & 1u);
-  return static_cast<uint16_t>(b >> 16);
+  const uint32_t b = __float_as_uint(f);
+  const uint32_t rounded = (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16;
+  const uint32_t quiet_nan = ((b >> 16) & 0x8000u) | 0x7FC0u;
+  return static_cast<uint16_t>((b & 0x7FFFFFFFu) > 0x7F800000u ? quiet_nan : rounded);
 }
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return __uint_as_float(static_cast<uint32_t>(h) << 16);
@@ -89,32 +94,55 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
 // ---- cross-lane ------------------------------------------------------------
 // Butterfly min / max over aligned groups of `span` lanes (span a power of two
 // <= 64).  Every lane of the group ends with the group's result.
-// The first three steps stay inside the VALU as DPP moves: quad_perm [1,0,3,2]
-// and [2,3,0,1] fold a quad, after which all four lanes of a quad agree, so the
-// half-row mirror (lane i <-> 7 - i) delivers "the other quad" to every lane.
-// Wider steps go through the LDS crossbar (__shfl_xor).
+//
+// The values travel as order-preserving integer keys (key(f) = bits ^ ((bits >>
+// 31) & 0x7FFFFFFF), an involution; -0 sorts below +0 as in v_min_f32): integer
+// min / max take a DPP operand directly, so a step is ONE instruction per
+// quantity, where the float forms need a move and two canonicalisations more.
+// Steps: quad_perm [1,0,3,2] and [2,3,0,1] fold a quad, after which the four
+// lanes of a quad agree, so the half-row mirror (lane i <-> 7 - i) delivers "the
+// other quad"; row_ror:8 delivers the other half of a 16-lane row; lanes 16
+// apart swap through ds_swizzle, lanes 32 apart through ds_bpermute.
+__device__ __forceinline__ int order_key(float f) {
+  const int b = __float_as_int(f);
+  return b ^ ((b >> 31) & 0x7FFFFFFF);
+}
+__device__ __forceinline__ float key_value(int k) { return __int_as_float(k ^ ((k >> 31) & 0x7FFFFFFF)); }
+
 template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, true);  // typed: keeps v's known-canonical status
+__device__ __forceinline__ int dpp_lanes(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, true);
 }
 
 __device__ __forceinline__ void group_minmax(float& mn, float& mx, int span) {
+  int lo = order_key(mn), hi = order_key(mx);
   if (span >= 2) {
-    mn = fminf(mn, dpp_move<0xB1>(mn));
-    mx = fmaxf(mx, dpp_move<0xB1>(mx));
+    lo = min(lo, dpp_lanes<0xB1>(lo));
+    hi = max(hi, dpp_lanes<0xB1>(hi));
   }
   if (span >= 4) {
-    mn = fminf(mn, dpp_move<0x4E>(mn));
-    mx = fmaxf(mx, dpp_move<0x4E>(mx));
+    lo = min(lo, dpp_lanes<0x4E>(lo));
+    hi = max(hi, dpp_lanes<0x4E>(hi));
   }
   if (span >= 8) {
-    mn = fminf(mn, dpp_move<0x141>(mn));
-    mx = fmaxf(mx, dpp_move<0x141>(mx));
+    lo = min(lo, dpp_lanes<0x141>(lo));
+    hi = max(hi, dpp_lanes<0x141>(hi));
   }
-  for (int m = 8; m < span; m <<= 1) {
-    mn = fminf(mn, __shfl_xor(mn, m));
-    mx = fmaxf(mx, __shfl_xor(mx, m));
+  if (span >= 16) {
+    lo = min(lo, dpp_lanes<0x128>(lo));
+    hi = max(hi, dpp_lanes<0x128>(hi));
   }
+  if (span >= 32) {
+    constexpr int kSwap16 = 0x401F;  // bit-mask mode: and 0x1F, or 0, xor 0x10
+    lo = min(lo, __builtin_amdgcn_ds_swizzle(lo, kSwap16));
+    hi = max(hi, __builtin_amdgcn_ds_swizzle(hi, kSwap16));
+  }
+  if (span >= 64) {
+    lo = min(lo, __shfl_xor(lo, 32));
+    hi = max(hi, __shfl_xor(hi, 32));
+  }
+  mn = key_value(lo);
+  mx = key_value(hi);
 }
 
 }  // namespace exact

@@ -306,7 +306,10 @@ struct Geometry {
 static Geometry plan_rows(int64_t G, int max_opt) {
   Geometry g;
   g.opr = static_cast<int>((G + 7) / 8);
-  int opt = (g.opr + 31) / 32;
+  // Aim for 16 lanes per row: the per-lane fixed work (row statistics butterfly,
+  // the scale division, parameter stores, address set-up) is then shared by
+  // two octs at 256 columns and four at 512, and a row never leaves one DPP row.
+  int opt = (g.opr + 15) / 16;
   if (opt > max_opt) opt = max_opt;
   if (opt == 3) opt = 4;
   if (opt < 1) opt = 1;
