@@ -172,3 +172,30 @@ def test_masks_random_sizes():
         y, mask = e.dropout_fwd(x, 0.3, None, seed, off)
         wy, wm = o.dropout_fwd(x, 0.3, o.philox_noise_flat(seed, off, n))
         assert np.array_equal(y.view(np.uint32), wy.view(np.uint32)) and np.array_equal(mask, wm), n
+
+
+def test_spmm_degenerate_row_layouts():
+    """Row layouts that stress the search for a chunk's first row: a single
+    row, only the last row filled, one hub row among empty ones, M around
+    multiples of the wavefront size."""
+    rng = np.random.default_rng(7)
+    for trial in range(60):
+        M = int(rng.choice([1, 2, 3, 63, 64, 65, 129, 1000, 4097]))
+        N, K = int(rng.integers(1, 40)), int(rng.choice([1, 4, 7, 64]))
+        mode = trial % 3
+        if mode == 0:
+            deg = rng.integers(0, 4, M)
+        elif mode == 1:
+            deg = np.zeros(M, np.int64)
+            deg[rng.integers(0, M)] = rng.integers(1, 400)
+        else:
+            deg = np.zeros(M, np.int64)
+            deg[-1], deg[0] = rng.integers(1, 200), rng.integers(0, 3)
+        rowptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+        col = rng.integers(0, N, int(rowptr[-1]))
+        val = rng.standard_normal(col.size).astype(np.float32)
+        X = rng.standard_normal((N, K)).astype(np.float32)
+        reduce = "sum" if trial % 2 else "mean"
+        got = e.spmm(rowptr, col, val, X, reduce, np.int32 if trial % 4 < 2 else np.int64)
+        want = o.spmm_csr(rowptr, col, val, X, reduce)
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * max(1.0, np.abs(want).max())), (trial, M, N, K, mode)
