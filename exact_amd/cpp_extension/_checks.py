@@ -1,7 +1,8 @@
 """Argument checks with the reference's error convention
 (exact/exact/cpp_extension/ext_common.h:2-27): RuntimeError with the same
 message for non-device, non-contiguous, wrong-rank or wrong-dtype tensors.
-The reference also admits float16; this library computes in fp32 only."""
+fp32 everywhere; fp16 where the library has fp16 kernels (pack / unpack and the
+mask activations), as the reference's AT_DISPATCH_FLOATING_TYPES_AND_HALF admits."""
 import torch
 
 
@@ -25,6 +26,14 @@ def check_device_tensor(t, name, dim=None, dtypes=(torch.float32,)):
         _fail(f"The dimension of {name} is not correct!")
     if t.dtype not in dtypes:
         _fail(f"The type of {name} is not correct!")
+
+
+FLOAT_OR_HALF = (torch.float32, torch.float16)
+
+
+def suffix(t):
+    """Entry-point suffix for the element type of t."""
+    return "f16" if t.dtype == torch.float16 else "f32"
 
 
 def stream_ptr(t):

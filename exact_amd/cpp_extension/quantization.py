@@ -14,7 +14,7 @@ from .. import _lib
 from ..conf import config
 from ..rng import next_philox
 from . import _checks
-from ._checks import check_device_tensor, ptr
+from ._checks import FLOAT_OR_HALF, check_device_tensor, ptr, suffix
 
 
 def packed_nbytes(N: int, G: int, bits: int) -> int:
@@ -64,14 +64,15 @@ def pack_single_precision(data, min, max, scale, bits, stochastic):  # noqa: A00
 def unpack_single_precision(data, bits, scale, min, N, group_size):  # noqa: A002
     """quantization.cc:50-62."""
     check_device_tensor(data, "data", 1, (torch.int8,))
-    check_device_tensor(scale, "scale", 1)
-    check_device_tensor(min, "min", 1)
+    check_device_tensor(scale, "scale", 1, FLOAT_OR_HALF)
+    check_device_tensor(min, "min", 1, (scale.dtype,))
     _check_bits(bits)
     N, G = int(N), int(group_size)
     if data.numel() < packed_nbytes(N, G, bits) - 1 or scale.numel() < N or min.numel() < N:
         raise RuntimeError("packed data / scale / min are too short for N x group_size")
-    out = torch.empty((N, G), dtype=scale.dtype, device=data.device)
-    rc = _lib.lib().exact_unpack_f32(ptr(data), bits, ptr(scale), ptr(min), N, G, ptr(out), _checks.stream_ptr(data))
+    out = torch.empty((N, G), dtype=scale.dtype, device=data.device)     # the dtype of scale decides, as at :209
+    unpack = getattr(_lib.lib(), "exact_unpack_" + suffix(scale))
+    rc = unpack(ptr(data), bits, ptr(scale), ptr(min), N, G, ptr(out), _checks.stream_ptr(data))
     _lib.check(rc, "unpack_single_precision")
     return out
 
@@ -81,11 +82,24 @@ def minmax_pack(data, bits, want_fp32=False):
     """One pass over data[N, G]: per-row min and scale (ops.py:39, 61-66),
     quantise + pack, and the bf16 copies of scale / min (ops.py:80-81).
     -> (packed int8, scale bf16, min bf16[, scale fp32, min fp32])."""
-    check_device_tensor(data, "data", 2)
+    check_device_tensor(data, "data", 2, FLOAT_OR_HALF)
     _check_bits(bits)
     N, G = data.shape
     dev = data.device
     packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=dev)
+    if data.dtype == torch.float16:
+        # fp16 activations: scale / min come back in fp16 (reference ops.py:82-83)
+        if G > 1024:
+            raise RuntimeError("fp16 activations: at most 1024 values per row")
+        scale_h = torch.empty(N, dtype=torch.float16, device=dev)
+        min_h = torch.empty(N, dtype=torch.float16, device=dev)
+        noise, seed, offset = _noise_for(data.shape, dev)
+        rc = _lib.lib().exact_minmax_pack_f16(ptr(data), ptr(noise), seed, offset, N, G, bits, ptr(packed),
+                                              ptr(scale_h), ptr(min_h), _checks.stream_ptr(data))
+        _lib.check(rc, "minmax_pack")
+        if want_fp32:
+            return packed, scale_h, min_h, scale_h.float(), min_h.float()
+        return packed, scale_h, min_h
     scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     need32 = want_fp32 or G > 1024
@@ -141,7 +155,7 @@ class ActQuantizedReLU(torch.autograd.Function):
         n = input.numel()
         out = torch.empty_like(input)
         mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
-        rc = _lib.lib().exact_relu_fwd_f32(ptr(input), n, ptr(out), ptr(mask), _checks.stream_ptr(input))
+        rc = getattr(_lib.lib(), "exact_relu_fwd_" + suffix(input))(ptr(input), n, ptr(out), ptr(mask), _checks.stream_ptr(input))
         _lib.check(rc, "act_quantized_relu")
         ctx.save_for_backward(mask)
         return out
@@ -151,7 +165,7 @@ class ActQuantizedReLU(torch.autograd.Function):
         (mask,) = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         grad_input = torch.empty_like(grad_output)
-        rc = _lib.lib().exact_relu_bwd_f32(ptr(grad_output), ptr(mask), grad_output.numel(),
+        rc = getattr(_lib.lib(), "exact_relu_bwd_" + suffix(grad_output))(ptr(grad_output), ptr(mask), grad_output.numel(),
                                            ptr(grad_input), _checks.stream_ptr(grad_output))
         _lib.check(rc, "act_quantized_relu backward")
         return grad_input
@@ -159,7 +173,7 @@ class ActQuantizedReLU(torch.autograd.Function):
 
 def act_quantized_relu(input):  # noqa: A002
     """quantization.cc:81-84."""
-    check_device_tensor(input, "input")
+    check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     return ActQuantizedReLU.apply(input)
 
 
@@ -171,7 +185,7 @@ class ActQuantizedLeakyReLU(torch.autograd.Function):
         n = input.numel()
         out = torch.empty_like(input)
         mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
-        rc = _lib.lib().exact_leaky_relu_fwd_f32(ptr(input), n, float(slope), ptr(out), ptr(mask),
+        rc = getattr(_lib.lib(), "exact_leaky_relu_fwd_" + suffix(input))(ptr(input), n, float(slope), ptr(out), ptr(mask),
                                                  _checks.stream_ptr(input))
         _lib.check(rc, "act_quantized_leaky_relu")
         ctx.save_for_backward(mask)
@@ -183,7 +197,7 @@ class ActQuantizedLeakyReLU(torch.autograd.Function):
         (mask,) = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         grad_input = torch.empty_like(grad_output)
-        rc = _lib.lib().exact_leaky_relu_bwd_f32(ptr(grad_output), ptr(mask), grad_output.numel(), ctx.slope,
+        rc = getattr(_lib.lib(), "exact_leaky_relu_bwd_" + suffix(grad_output))(ptr(grad_output), ptr(mask), grad_output.numel(), ctx.slope,
                                                  ptr(grad_input), _checks.stream_ptr(grad_output))
         _lib.check(rc, "act_quantized_leaky_relu backward")
         return grad_input, None
@@ -191,7 +205,7 @@ class ActQuantizedLeakyReLU(torch.autograd.Function):
 
 def act_quantized_leaky_relu(input, slope):  # noqa: A002
     """quantization.cc:105-108."""
-    check_device_tensor(input, "input")
+    check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     return ActQuantizedLeakyReLU.apply(input, slope)
 
 
@@ -206,7 +220,7 @@ class ActQuantizedDropout(torch.autograd.Function):
         out = torch.empty_like(input)
         mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
         noise, seed, offset = _noise_for(input.shape, input.device)
-        rc = _lib.lib().exact_dropout_fwd_f32(ptr(input), ptr(noise), seed, offset, float(p), n,
+        rc = getattr(_lib.lib(), "exact_dropout_fwd_" + suffix(input))(ptr(input), ptr(noise), seed, offset, float(p), n,
                                               ptr(out), ptr(mask), _checks.stream_ptr(input))
         _lib.check(rc, "act_quantized_dropout")
         ctx.save_for_backward(mask)
@@ -221,7 +235,7 @@ class ActQuantizedDropout(torch.autograd.Function):
         (mask,) = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         grad_input = torch.empty_like(grad_output)
-        rc = _lib.lib().exact_dropout_bwd_f32(ptr(grad_output), ptr(mask), ctx.p, grad_output.numel(),
+        rc = getattr(_lib.lib(), "exact_dropout_bwd_" + suffix(grad_output))(ptr(grad_output), ptr(mask), ctx.p, grad_output.numel(),
                                               ptr(grad_input), _checks.stream_ptr(grad_output))
         _lib.check(rc, "act_quantized_dropout backward")
         return grad_input, None, None
@@ -229,7 +243,7 @@ class ActQuantizedDropout(torch.autograd.Function):
 
 def act_quantized_dropout(input, p, train):  # noqa: A002
     """quantization.cc:131-134."""
-    check_device_tensor(input, "input")
+    check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     if not train:
         return input                      # quantization.cc:115-117
     return ActQuantizedDropout.apply(input, p, train)
@@ -244,12 +258,12 @@ def fusable_width(G: int) -> bool:
 def relu_dropout_fwd(input, p):  # noqa: A002
     """dropout(relu(input)) in one pass -> (output, joint 1-bit mask); the
     gradient of the pair is dropout_bwd on that mask."""
-    check_device_tensor(input, "input")
+    check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     n = input.numel()
     out = torch.empty_like(input)
     mask = torch.empty(mask_nwords(n), dtype=torch.int32, device=input.device)
     noise, seed, offset = _noise_for(input.shape, input.device)
-    rc = _lib.lib().exact_relu_dropout_fwd_f32(ptr(input), ptr(noise), seed, offset, float(p), n, ptr(out), ptr(mask),
+    rc = getattr(_lib.lib(), "exact_relu_dropout_fwd_" + suffix(input))(ptr(input), ptr(noise), seed, offset, float(p), n, ptr(out), ptr(mask),
                                                _checks.stream_ptr(input))
     _lib.check(rc, "relu_dropout")
     return out, mask
@@ -282,9 +296,9 @@ def relu_dropout_minmax_pack(input, p, bits):  # noqa: A002
 def dropout_bwd(grad_output, mask, p):
     """dx = bit ? dy / (1 - p) : 0 (quantization_cuda_kernel.cu:565-569)."""
     grad_output = grad_output.contiguous()
-    check_device_tensor(grad_output, "grad_output")
+    check_device_tensor(grad_output, "grad_output", None, FLOAT_OR_HALF)
     grad_input = torch.empty_like(grad_output)
-    rc = _lib.lib().exact_dropout_bwd_f32(ptr(grad_output), ptr(mask), float(p), grad_output.numel(),
+    rc = getattr(_lib.lib(), "exact_dropout_bwd_" + suffix(grad_output))(ptr(grad_output), ptr(mask), float(p), grad_output.numel(),
                                           ptr(grad_input), _checks.stream_ptr(grad_output))
     _lib.check(rc, "dropout backward")
     return grad_input

@@ -29,6 +29,9 @@ def spmm_csr(rowptr, col, value, mat, reduce):
     {sum, mean} (spmm_cuda.cu:106-170)."""
     if reduce not in REDUCE:
         raise NotImplementedError(f"reduce='{reduce}': use spmm_max_fw / spmm_min_fw for max and min")
+    if isinstance(mat, torch.Tensor) and mat.dtype == torch.float16:
+        # fp16 activations (autocast): gather and accumulate in fp32, round the result once
+        return spmm_csr(rowptr, col, value, mat.float(), reduce).to(torch.float16)
     _check_index(rowptr, "rowptr")
     _check_index(col, "col")
     if not _checks.on_device(mat):
@@ -103,7 +106,9 @@ def _csc_operands(kind, row, value, rowcount, csr2csc, has_value, dtype):
     key = (kind, row.data_ptr(), csr2csc.data_ptr(), row.numel(),
            value.data_ptr() if has_value else 0, value._version if has_value else 0,
            rowcount.data_ptr() if rowcount is not None else 0)
-    hit = _CSC_CACHE.get(key)
+    # fp16 values are per-call copies made by autocast: nothing to reuse, nothing to keep
+    cacheable = not (has_value and value.dtype != torch.float32)
+    hit = _CSC_CACHE.get(key) if cacheable else None
     if hit is not None:
         _CSC_CACHE.move_to_end(key)
         return hit[0], hit[1]
@@ -111,8 +116,10 @@ def _csc_operands(kind, row, value, rowcount, csr2csc, has_value, dtype):
     if kind == "sum":
         w = value.detach().index_select(0, csr2csc) if has_value else None
     else:
-        cnt = rowcount.to(dtype).index_select(0, row_csc).clamp_(min=1)
+        cnt = rowcount.to(torch.float32).index_select(0, row_csc).clamp_(min=1)   # fp32 whatever `dtype` is
         w = value.detach().index_select(0, csr2csc).div(cnt) if has_value else cnt.pow_(-1)
+    if not cacheable:
+        return row_csc, w
     # the inputs are kept alive with the entry so their addresses cannot be reused
     _CSC_CACHE[key] = (row_csc, w, (row, value, rowcount, csr2csc))
     while len(_CSC_CACHE) > _CSC_CACHE_MAX:
@@ -134,6 +141,8 @@ def spmm_value_bw(row, rowptr, col, mat, grad, reduce):
     edge values, out[e] = mat[col[e]] . grad[row[e]] (/ row length for mean)."""
     if reduce not in REDUCE:
         raise NotImplementedError(f"reduce='{reduce}'")
+    if torch.float16 in (mat.dtype, grad.dtype):
+        return spmm_value_bw(row, rowptr, col, mat.float(), grad.float(), reduce).to(torch.float16)
     for t, name in ((row, "row"), (rowptr, "rowptr"), (col, "col")):
         _check_index(t, name)
     for t, name in ((mat, "mat"), (grad, "grad")):
@@ -181,6 +190,9 @@ def spmm_mean_bw(row, rowptr, col, value, rowcount, colptr, csr2csc, mat, grad_o
 # ---- max / min aggregation ----------------------------------------------------
 def _spmm_extreme_fw(rowptr, col, value, mat, is_max):
     """spmm_max_fw / spmm_min_fw (spmm.cc:145-157, 199-212) -> (out, arg_out)."""
+    if isinstance(mat, torch.Tensor) and mat.dtype == torch.float16:
+        out, arg = _spmm_extreme_fw(rowptr, col, value, mat.float(), is_max)
+        return out.to(torch.float16), arg
     _check_index(rowptr, "rowptr")
     _check_index(col, "col")
     if not _checks.on_device(mat):

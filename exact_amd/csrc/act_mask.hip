@@ -23,6 +23,11 @@ namespace exact {
 
 constexpr int kTileQuads = 2 * kBlock;  // quads per workgroup
 
+// Element type T is float or half_t (fp16: the reference instantiates these
+// kernels for at::Half as well; values are widened to fp32 on load and rounded
+// to fp16 once on store, which is what at::Half arithmetic amounts to here).
+typedef half_t half4_t __attribute__((ext_vector_type(4)));
+
 template <bool VEC4>
 __device__ __forceinline__ void load4(const float* __restrict__ p, int nv, float (&v)[4]) {
   if (VEC4 && nv == 4) {
@@ -31,6 +36,17 @@ __device__ __forceinline__ void load4(const float* __restrict__ p, int nv, float
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = (i < nv) ? p[i] : 0.f;
+  }
+}
+template <bool VEC4>
+__device__ __forceinline__ void load4(const half_t* __restrict__ p, int nv, float (&v)[4]) {
+  if (VEC4 && nv == 4) {
+    const half4_t a = __builtin_nontemporal_load(reinterpret_cast<const half4_t*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<float>(a[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (i < nv) ? static_cast<float>(p[i]) : 0.f;
   }
 }
 
@@ -42,6 +58,18 @@ __device__ __forceinline__ void store4(float* __restrict__ p, int nv, const floa
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       if (i < nv) p[i] = v[i];
+  }
+}
+template <bool VEC4>
+__device__ __forceinline__ void store4(half_t* __restrict__ p, int nv, const float (&v)[4]) {
+  if (VEC4 && nv == 4) {
+    const half4_t a = {static_cast<half_t>(v[0]), static_cast<half_t>(v[1]), static_cast<half_t>(v[2]),
+                       static_cast<half_t>(v[3])};
+    __builtin_nontemporal_store(a, reinterpret_cast<half4_t*>(p));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < nv) p[i] = static_cast<half_t>(v[i]);
   }
 }
 
@@ -71,9 +99,9 @@ __device__ __forceinline__ uint32_t load_mask_nibble(const uint32_t* __restrict_
   return (mask[quad >> 3] >> (4 * (quad & 7))) & 0xFu;
 }
 
-template <bool VEC4>
-__global__ __launch_bounds__(kBlock) void relu_fwd_kernel(const float* __restrict__ x, int64_t n,
-                                                          float* __restrict__ y,
+template <bool VEC4, typename T>
+__global__ __launch_bounds__(kBlock) void relu_fwd_kernel(const T* __restrict__ x, int64_t n,
+                                                          T* __restrict__ y,
                                                           uint32_t* __restrict__ mask) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -95,10 +123,10 @@ __global__ __launch_bounds__(kBlock) void relu_fwd_kernel(const float* __restric
   }
 }
 
-template <bool VEC4>
-__global__ __launch_bounds__(kBlock) void relu_bwd_kernel(const float* __restrict__ dy,
+template <bool VEC4, typename T>
+__global__ __launch_bounds__(kBlock) void relu_bwd_kernel(const T* __restrict__ dy,
                                                           const uint32_t* __restrict__ mask, int64_t n,
-                                                          float* __restrict__ dx) {
+                                                          T* __restrict__ dx) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
@@ -115,9 +143,9 @@ __global__ __launch_bounds__(kBlock) void relu_bwd_kernel(const float* __restric
 
 // LeakyReLU with the same 1-bit mask (quantization_cuda_kernel.cu:339-371, 395-412):
 // y = x > 0 ? x : x * slope; dx = bit ? dy : dy * slope.
-template <bool VEC4>
-__global__ __launch_bounds__(kBlock) void leaky_relu_fwd_kernel(const float* __restrict__ x, int64_t n, float slope,
-                                                                float* __restrict__ y,
+template <bool VEC4, typename T>
+__global__ __launch_bounds__(kBlock) void leaky_relu_fwd_kernel(const T* __restrict__ x, int64_t n, float slope,
+                                                                T* __restrict__ y,
                                                                 uint32_t* __restrict__ mask) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -139,10 +167,10 @@ __global__ __launch_bounds__(kBlock) void leaky_relu_fwd_kernel(const float* __r
   }
 }
 
-template <bool VEC4>
-__global__ __launch_bounds__(kBlock) void leaky_relu_bwd_kernel(const float* __restrict__ dy,
+template <bool VEC4, typename T>
+__global__ __launch_bounds__(kBlock) void leaky_relu_bwd_kernel(const T* __restrict__ dy,
                                                                 const uint32_t* __restrict__ mask, int64_t n,
-                                                                float slope, float* __restrict__ dx) {
+                                                                float slope, T* __restrict__ dx) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
@@ -160,12 +188,12 @@ __global__ __launch_bounds__(kBlock) void leaky_relu_bwd_kernel(const float* __r
 // RELU: the input first goes through ReLU and the mask bit is (x > 0) && keep --
 // ReLU followed by dropout in one pass, with one mask for the pair (the
 // backward of the pair is dx = bit ? dy / (1 - p) : 0, i.e. dropout_bwd_kernel).
-template <bool VEC4, bool NOISE_IN, bool RELU>
-__global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const float* __restrict__ x,
+template <bool VEC4, bool NOISE_IN, bool RELU, typename T>
+__global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const T* __restrict__ x,
                                                              const float* __restrict__ noise,
                                                              uint32_t seed_lo, uint32_t seed_hi,
                                                              uint32_t off_lo, uint32_t off_hi, float p,
-                                                             float pinv, int64_t n, float* __restrict__ y,
+                                                             float pinv, int64_t n, T* __restrict__ y,
                                                              uint32_t* __restrict__ mask) {
   const int64_t qa = static_cast<int64_t>(blockIdx.x) * kTileQuads + threadIdx.x;
   const int64_t qb = qa + kBlock;
@@ -211,10 +239,10 @@ __global__ __launch_bounds__(kBlock) void dropout_fwd_kernel(const float* __rest
   }
 }
 
-template <bool VEC4>
-__global__ __launch_bounds__(kBlock) void dropout_bwd_kernel(const float* __restrict__ dy,
+template <bool VEC4, typename T>
+__global__ __launch_bounds__(kBlock) void dropout_bwd_kernel(const T* __restrict__ dy,
                                                              const uint32_t* __restrict__ mask, float p1m,
-                                                             int64_t n, float* __restrict__ dx) {
+                                                             int64_t n, T* __restrict__ dx) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
@@ -229,6 +257,9 @@ __global__ __launch_bounds__(kBlock) void dropout_bwd_kernel(const float* __rest
   }
 }
 
+// a quad of T is one aligned vector access
+template <typename T>
+static bool quad_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & (4 * sizeof(T) - 1)) == 0; }
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static dim3 tile_grid(int64_t n) {
@@ -236,14 +267,64 @@ static dim3 tile_grid(int64_t n) {
   return dim3(static_cast<unsigned>((quads + kTileQuads - 1) / kTileQuads));
 }
 
-}  // namespace exact
+static int check_n(int64_t n) { return (n < 0 || n > (int64_t{1} << 40)) ? EXACT_E_SHAPE : EXACT_OK; }
 
-using namespace exact;
+template <typename T>
+static int relu_forward(const T* x, int64_t n, T* y, uint32_t* mask, void* stream) {
+  if (int rc = check_n(n)) return rc;
+  if (n == 0) return EXACT_OK;
+  if (!x || !y || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (quad_aligned<T>(x) && quad_aligned<T>(y))
+    hipLaunchKernelGGL((relu_fwd_kernel<true, T>), tile_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
+  else
+    hipLaunchKernelGGL((relu_fwd_kernel<false, T>), tile_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
+  return launch_status();
+}
 
-template <bool RELU>
-static int dropout_forward(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p, int64_t n,
-                           float* y, uint32_t* mask, void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+template <typename T>
+static int relu_backward(const T* dy, const uint32_t* mask, int64_t n, T* dx, void* stream) {
+  if (int rc = check_n(n)) return rc;
+  if (n == 0) return EXACT_OK;
+  if (!dy || !dx || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (quad_aligned<T>(dy) && quad_aligned<T>(dx))
+    hipLaunchKernelGGL((relu_bwd_kernel<true, T>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
+  else
+    hipLaunchKernelGGL((relu_bwd_kernel<false, T>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
+  return launch_status();
+}
+
+template <typename T>
+static int leaky_forward(const T* x, int64_t n, float slope, T* y, uint32_t* mask, void* stream) {
+  if (int rc = check_n(n)) return rc;
+  if (n == 0) return EXACT_OK;
+  if (!x || !y || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (quad_aligned<T>(x) && quad_aligned<T>(y))
+    hipLaunchKernelGGL((leaky_relu_fwd_kernel<true, T>), tile_grid(n), dim3(kBlock), 0, s, x, n, slope, y, mask);
+  else
+    hipLaunchKernelGGL((leaky_relu_fwd_kernel<false, T>), tile_grid(n), dim3(kBlock), 0, s, x, n, slope, y, mask);
+  return launch_status();
+}
+
+template <typename T>
+static int leaky_backward(const T* dy, const uint32_t* mask, int64_t n, float slope, T* dx, void* stream) {
+  if (int rc = check_n(n)) return rc;
+  if (n == 0) return EXACT_OK;
+  if (!dy || !dx || !mask) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (quad_aligned<T>(dy) && quad_aligned<T>(dx))
+    hipLaunchKernelGGL((leaky_relu_bwd_kernel<true, T>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, slope, dx);
+  else
+    hipLaunchKernelGGL((leaky_relu_bwd_kernel<false, T>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, slope, dx);
+  return launch_status();
+}
+
+template <bool RELU, typename T>
+static int dropout_forward(const T* x, const float* noise, uint64_t seed, uint64_t offset, float p, int64_t n,
+                           T* y, uint32_t* mask, void* stream) {
+  if (int rc = check_n(n)) return rc;
   if (!(p >= 0.f && p < 1.f)) return EXACT_E_ARG;
   if (n == 0) return EXACT_OK;
   if (!x || !y || !mask) return EXACT_E_NULL;
@@ -252,93 +333,95 @@ static int dropout_forward(const float* x, const float* noise, uint64_t seed, ui
   const float pinv = static_cast<float>(1.0 / (1.0 - static_cast<double>(p)));
   const uint32_t sl = static_cast<uint32_t>(seed), sh = static_cast<uint32_t>(seed >> 32);
   const uint32_t ol = static_cast<uint32_t>(offset), oh = static_cast<uint32_t>(offset >> 32);
-  const bool v4 = aligned16(x) && aligned16(y) && (!noise || aligned16(noise));
+  const bool v4 = quad_aligned<T>(x) && quad_aligned<T>(y) && (!noise || aligned16(noise));
   const dim3 grid = tile_grid(n);
   if (noise) {
-    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, true, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
-    else hipLaunchKernelGGL((dropout_fwd_kernel<false, true, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, true, RELU, T>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+    else hipLaunchKernelGGL((dropout_fwd_kernel<false, true, RELU, T>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
   } else {
-    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, false, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
-    else hipLaunchKernelGGL((dropout_fwd_kernel<false, false, RELU>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+    if (v4) hipLaunchKernelGGL((dropout_fwd_kernel<true, false, RELU, T>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
+    else hipLaunchKernelGGL((dropout_fwd_kernel<false, false, RELU, T>), grid, dim3(kBlock), 0, s, x, noise, sl, sh, ol, oh, p, pinv, n, y, mask);
   }
   return launch_status();
 }
 
-extern "C" {
-
-int exact_relu_fwd_f32(const float* x, int64_t n, float* y, uint32_t* mask, void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
-  if (n == 0) return EXACT_OK;
-  if (!x || !y || !mask) return EXACT_E_NULL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (aligned16(x) && aligned16(y))
-    hipLaunchKernelGGL((relu_fwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
-  else
-    hipLaunchKernelGGL((relu_fwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, x, n, y, mask);
-  return launch_status();
-}
-
-int exact_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float* dx, void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
-  if (n == 0) return EXACT_OK;
-  if (!dy || !dx || !mask) return EXACT_E_NULL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (aligned16(dy) && aligned16(dx))
-    hipLaunchKernelGGL((relu_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
-  else
-    hipLaunchKernelGGL((relu_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, dx);
-  return launch_status();
-}
-
-int exact_leaky_relu_fwd_f32(const float* x, int64_t n, float slope, float* y, uint32_t* mask, void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
-  if (n == 0) return EXACT_OK;
-  if (!x || !y || !mask) return EXACT_E_NULL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (aligned16(x) && aligned16(y))
-    hipLaunchKernelGGL((leaky_relu_fwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, x, n, slope, y, mask);
-  else
-    hipLaunchKernelGGL((leaky_relu_fwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, x, n, slope, y, mask);
-  return launch_status();
-}
-
-int exact_leaky_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float slope, float* dx,
-                             void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
-  if (n == 0) return EXACT_OK;
-  if (!dy || !dx || !mask) return EXACT_E_NULL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (aligned16(dy) && aligned16(dx))
-    hipLaunchKernelGGL((leaky_relu_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, slope, dx);
-  else
-    hipLaunchKernelGGL((leaky_relu_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, n, slope, dx);
-  return launch_status();
-}
-
-int exact_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p,
-                          int64_t n, float* y, uint32_t* mask, void* stream) {
-  return dropout_forward<false>(x, noise, seed, offset, p, n, y, mask, stream);
-}
-
-int exact_relu_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p,
-                               int64_t n, float* y, uint32_t* mask, void* stream) {
-  return dropout_forward<true>(x, noise, seed, offset, p, n, y, mask, stream);
-}
-
-int exact_dropout_bwd_f32(const float* dy, const uint32_t* mask, float p, int64_t n, float* dx,
-                          void* stream) {
-  if (n < 0 || n > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+template <typename T>
+static int dropout_backward(const T* dy, const uint32_t* mask, float p, int64_t n, T* dx, void* stream) {
+  if (int rc = check_n(n)) return rc;
   if (!(p >= 0.f && p < 1.f)) return EXACT_E_ARG;
   if (n == 0) return EXACT_OK;
   if (!dy || !dx || !mask) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   // quantization.cc:121,127: p1m = 1. - p stored as double, read back into a float
   const float p1m = static_cast<float>(1.0 - static_cast<double>(p));
-  if (aligned16(dy) && aligned16(dx))
-    hipLaunchKernelGGL((dropout_bwd_kernel<true>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
+  if (quad_aligned<T>(dy) && quad_aligned<T>(dx))
+    hipLaunchKernelGGL((dropout_bwd_kernel<true, T>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
   else
-    hipLaunchKernelGGL((dropout_bwd_kernel<false>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
+    hipLaunchKernelGGL((dropout_bwd_kernel<false, T>), tile_grid(n), dim3(kBlock), 0, s, dy, mask, p1m, n, dx);
   return launch_status();
+}
+
+}  // namespace exact
+
+using namespace exact;
+
+static const half_t* hp(const uint16_t* p) { return reinterpret_cast<const half_t*>(p); }
+static half_t* hp(uint16_t* p) { return reinterpret_cast<half_t*>(p); }
+
+extern "C" {
+
+int exact_relu_fwd_f32(const float* x, int64_t n, float* y, uint32_t* mask, void* stream) {
+  return relu_forward<float>(x, n, y, mask, stream);
+}
+int exact_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float* dx, void* stream) {
+  return relu_backward<float>(dy, mask, n, dx, stream);
+}
+int exact_leaky_relu_fwd_f32(const float* x, int64_t n, float slope, float* y, uint32_t* mask, void* stream) {
+  return leaky_forward<float>(x, n, slope, y, mask, stream);
+}
+int exact_leaky_relu_bwd_f32(const float* dy, const uint32_t* mask, int64_t n, float slope, float* dx,
+                             void* stream) {
+  return leaky_backward<float>(dy, mask, n, slope, dx, stream);
+}
+int exact_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p,
+                          int64_t n, float* y, uint32_t* mask, void* stream) {
+  return dropout_forward<false, float>(x, noise, seed, offset, p, n, y, mask, stream);
+}
+int exact_relu_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset, float p,
+                               int64_t n, float* y, uint32_t* mask, void* stream) {
+  return dropout_forward<true, float>(x, noise, seed, offset, p, n, y, mask, stream);
+}
+int exact_dropout_bwd_f32(const float* dy, const uint32_t* mask, float p, int64_t n, float* dx,
+                          void* stream) {
+  return dropout_backward<float>(dy, mask, p, n, dx, stream);
+}
+
+// fp16 activations: the same kernels instantiated for 16-bit elements
+int exact_relu_fwd_f16(const uint16_t* x, int64_t n, uint16_t* y, uint32_t* mask, void* stream) {
+  return relu_forward<half_t>(hp(x), n, hp(y), mask, stream);
+}
+int exact_relu_bwd_f16(const uint16_t* dy, const uint32_t* mask, int64_t n, uint16_t* dx, void* stream) {
+  return relu_backward<half_t>(hp(dy), mask, n, hp(dx), stream);
+}
+int exact_leaky_relu_fwd_f16(const uint16_t* x, int64_t n, float slope, uint16_t* y, uint32_t* mask,
+                             void* stream) {
+  return leaky_forward<half_t>(hp(x), n, slope, hp(y), mask, stream);
+}
+int exact_leaky_relu_bwd_f16(const uint16_t* dy, const uint32_t* mask, int64_t n, float slope, uint16_t* dx,
+                             void* stream) {
+  return leaky_backward<half_t>(hp(dy), mask, n, slope, hp(dx), stream);
+}
+int exact_dropout_fwd_f16(const uint16_t* x, const float* noise, uint64_t seed, uint64_t offset, float p,
+                          int64_t n, uint16_t* y, uint32_t* mask, void* stream) {
+  return dropout_forward<false, half_t>(hp(x), noise, seed, offset, p, n, hp(y), mask, stream);
+}
+int exact_relu_dropout_fwd_f16(const uint16_t* x, const float* noise, uint64_t seed, uint64_t offset, float p,
+                               int64_t n, uint16_t* y, uint32_t* mask, void* stream) {
+  return dropout_forward<true, half_t>(hp(x), noise, seed, offset, p, n, hp(y), mask, stream);
+}
+int exact_dropout_bwd_f16(const uint16_t* dy, const uint32_t* mask, float p, int64_t n, uint16_t* dx,
+                          void* stream) {
+  return dropout_backward<half_t>(hp(dy), mask, p, n, hp(dx), stream);
 }
 
 }  // extern "C"

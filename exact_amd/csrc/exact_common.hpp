@@ -91,6 +91,17 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return __uint_as_float(static_cast<uint32_t>(h) << 16);
 }
 
+// ---- fp16 ------------------------------------------------------------------
+// IEEE binary16 with round-to-nearest-even conversions, as at::Half has them.
+using half_t = _Float16;
+__device__ __forceinline__ float round_to_half(float x) { return static_cast<float>(static_cast<half_t>(x)); }
+__device__ __forceinline__ uint16_t half_bits(float x) {
+  const half_t h = static_cast<half_t>(x);
+  uint16_t b;
+  __builtin_memcpy(&b, &h, 2);
+  return b;
+}
+
 // ---- cross-lane ------------------------------------------------------------
 // Butterfly min / max over aligned groups of `span` lanes (span a power of two
 // <= 64).  Every lane of the group ends with the group's result.

@@ -53,6 +53,23 @@ __device__ __forceinline__ void store_oct(float* __restrict__ p, int nv, const f
   }
 }
 
+// fp16 activations (the reference's kernels are also instantiated for at::Half,
+// quantization_cuda_kernel.cu:132-150): one oct is 16 bytes.  VEC == 4 here
+// means "whole octs, 16-byte aligned" (G % 8 == 0).
+template <int VEC, bool FULL>
+__device__ __forceinline__ void load_oct_half(const half_t* __restrict__ p, int nv, float (&v)[8]) {
+  if constexpr (VEC == 4) {
+    typedef half_t half8 __attribute__((ext_vector_type(8)));
+    half8 q = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (FULL || nv > 0) q = __builtin_nontemporal_load(reinterpret_cast<const half8*>(p));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = static_cast<float>(q[i]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (i < nv) ? static_cast<float>(__builtin_nontemporal_load(p + i)) : 0.f;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // pack
 // ---------------------------------------------------------------------------
@@ -89,7 +106,14 @@ struct PackArgs {
 // result -- "ReLU -> dropout -> quantize_activation of the next layer's input"
 // in one pass.  Needs G % 8 == 0, so that an oct is one Philox block and one
 // mask byte.
-template <int BITS, int OPT, int VEC, bool FULL, bool NOISE_IN, bool FUSED, bool ACT = false>
+//
+// HALF: x holds fp16 values and the 16-bit parameter outputs receive fp16 bits.
+// The arithmetic follows what the reference's at::Half instantiation computes:
+// at::Half operators evaluate in fp32 and round the result to fp16, so
+// (x - min) and its product with scale are each rounded to fp16, the noise is
+// then added in fp32 (quantization_cuda_kernel.cu:88-89); torch evaluates the
+// scale as (mx - mn).reciprocal() * B with an fp16 rounding after every step.
+template <int BITS, int OPT, int VEC, bool FULL, bool NOISE_IN, bool FUSED, bool ACT = false, bool HALF = false>
 __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   constexpr int WPT = 8 / BITS;
   constexpr float B = static_cast<float>((1 << BITS) - 1);
@@ -116,7 +140,8 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[k][i] = 0.f;
     } else {
-      load_oct<VEC, FULL>(a.x + row_off + d0, nv[k], v[k]);
+      if constexpr (HALF) load_oct_half<VEC, FULL>(reinterpret_cast<const half_t*>(a.x) + row_off + d0, nv[k], v[k]);
+      else load_oct<VEC, FULL>(a.x + row_off + d0, nv[k], v[k]);
     }
     if constexpr (ACT) {
       if (nv[k] > 0) {  // G % 8 == 0: a whole oct or nothing
@@ -163,13 +188,18 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
     mnv = lo;
     // ops.py:39 `(2 ** bits - 1) / (mx - mn)`: torch evaluates int / tensor as
     // tensor.reciprocal() * int, so two roundings
-    const float recip = 1.0f / (hi - lo);
-    sc = recip * B;
+    if constexpr (HALF) {
+      const float recip = round_to_half(1.0f / round_to_half(hi - lo));
+      sc = round_to_half(recip * B);
+    } else {
+      const float recip = 1.0f / (hi - lo);
+      sc = recip * B;
+    }
     if (row_ok && lane_in_row == 0) {
       if (a.scale_f32) a.scale_f32[n] = sc;
       if (a.min_f32) a.min_f32[n] = mnv;
-      if (a.scale_bf16) a.scale_bf16[n] = f32_to_bf16_rne(sc);
-      if (a.min_bf16) a.min_bf16[n] = f32_to_bf16_rne(mnv);
+      if (a.scale_bf16) a.scale_bf16[n] = HALF ? half_bits(sc) : f32_to_bf16_rne(sc);
+      if (a.min_bf16) a.min_bf16[n] = HALF ? half_bits(mnv) : f32_to_bf16_rne(mnv);
     }
   } else {
     if (row_ok) {
@@ -200,7 +230,9 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
     for (int i = 0; i < 8; ++i) {
       // quantization_cuda_kernel.cu:89, one rounding per operation
       float tq = v[k][i] - mnv;
+      if constexpr (HALF) tq = round_to_half(tq);
       tq = tq * sc;
+      if constexpr (HALF) tq = round_to_half(tq);
       tq = tq + u[i];
       tq = tq - 0.5f;
       tq = fmaxf(tq, 0.f);
@@ -457,6 +489,34 @@ static void launch_act_bits(const PackArgs& a, int bits, int opt, bool full, dim
   }
 }
 
+// ---- fp16 activations (HALF form): statistics + pack in one launch, G <= 1024 --
+template <int BITS, int OPT, bool NOISE_IN>
+static void launch_half_variant(const PackArgs& a, bool whole, bool full, dim3 grid, hipStream_t s) {
+  if (whole && full)
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, true, NOISE_IN, true, false, true>), grid, dim3(kBlock), 0, s, a);
+  else if (whole)
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, false, NOISE_IN, true, false, true>), grid, dim3(kBlock), 0, s, a);
+  else
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 1, false, NOISE_IN, true, false, true>), grid, dim3(kBlock), 0, s, a);
+}
+
+template <int BITS, bool NOISE_IN>
+static void launch_half_opt(const PackArgs& a, int opt, bool whole, bool full, dim3 grid, hipStream_t s) {
+  if (opt == 4) return launch_half_variant<BITS, 4, NOISE_IN>(a, whole, full, grid, s);
+  if (opt == 2) return launch_half_variant<BITS, 2, NOISE_IN>(a, whole, full, grid, s);
+  launch_half_variant<BITS, 1, NOISE_IN>(a, whole, full, grid, s);
+}
+
+template <bool NOISE_IN>
+static void launch_half_bits(const PackArgs& a, int bits, int opt, bool whole, bool full, dim3 grid, hipStream_t s) {
+  switch (bits) {
+    case 1: return launch_half_opt<1, NOISE_IN>(a, opt, whole, full, grid, s);
+    case 2: return launch_half_opt<2, NOISE_IN>(a, opt, whole, full, grid, s);
+    case 4: return launch_half_opt<4, NOISE_IN>(a, opt, whole, full, grid, s);
+    default: return launch_half_opt<8, NOISE_IN>(a, opt, whole, full, grid, s);
+  }
+}
+
 }  // namespace exact
 
 using namespace exact;
@@ -557,6 +617,46 @@ int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act
   const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), 1u);
   if (noise) launch_act_bits<true>(a, bits, g.opt, g.full, grid, s);
   else launch_act_bits<false>(a, bits, g.opt, g.full, grid, s);
+  return launch_status();
+}
+
+int exact_minmax_pack_f16(const uint16_t* x, const float* noise, uint64_t seed, uint64_t offset, int64_t N,
+                          int64_t G, int bits, uint8_t* packed, uint16_t* scale_f16, uint16_t* min_f16,
+                          void* stream) {
+  if (int rc = check_quant_shape(N, G, bits)) return rc;
+  if (G > 1024) return EXACT_E_SHAPE;
+  if (!packed) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t pad_index = exact_packed_nbytes(N, G, bits) - 1;
+  if (N == 0 || G == 0) {
+    hipLaunchKernelGGL(zero_byte_kernel, dim3(1), dim3(1), 0, s, packed + pad_index);
+    return launch_status();
+  }
+  if (!x) return EXACT_E_NULL;
+  if (!aligned(x, 2)) return EXACT_E_ALIGN;
+  const Geometry g = plan_rows(G, 4);
+  PackArgs a{};
+  a.x = reinterpret_cast<const float*>(x);  // the HALF form reads it as fp16
+  a.noise = noise;
+  a.seed_lo = static_cast<uint32_t>(seed);
+  a.seed_hi = static_cast<uint32_t>(seed >> 32);
+  a.off_lo = static_cast<uint32_t>(offset);
+  a.off_hi = static_cast<uint32_t>(offset >> 32);
+  a.N = N;
+  a.G = static_cast<int>(G);
+  a.opr = g.opr;
+  a.lpr_log2 = g.lpr_log2;
+  a.packed = packed;
+  a.pad_index = pad_index;
+  a.scale_bf16 = scale_f16;
+  a.min_bf16 = min_f16;
+  a.out_vec = (G % 8 == 0 && aligned(packed, 8)) ? 8 : (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
+  // whole octs: 16-byte loads of x (and of supplied fp32 noise)
+  const bool whole = (G % 8 == 0) && aligned(x, 16) && (!noise || aligned(noise, 16));
+  const int rows_per_wg = kBlock >> g.lpr_log2;
+  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), 1u);
+  if (noise) launch_half_bits<true>(a, bits, g.opt, whole, g.full && whole, grid, s);
+  else launch_half_bits<false>(a, bits, g.opt, whole, g.full && whole, grid, s);
   return launch_status();
 }
 

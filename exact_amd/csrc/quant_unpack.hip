@@ -53,8 +53,33 @@ __device__ __forceinline__ float exact_quotient(float q, float s, float r) {
   return __fmaf_rn(e, r, y);
 }
 
-template <int BITS, int SLOTS, int VEC, bool BF16P>
+// How scale / min (and, for fp16, the output) are stored.
+enum ParamKind { kParamF32 = 0, kParamBF16 = 1, kParamF16 = 2 };
+
+template <int VEC>
+__device__ __forceinline__ void store_quad_half(half_t* __restrict__ p, int nv, const float (&v)[4]) {
+  if constexpr (VEC == 4) {
+    typedef half_t half4 __attribute__((ext_vector_type(4)));
+    if (nv > 0) {
+      const half4 q = {static_cast<half_t>(v[0]), static_cast<half_t>(v[1]), static_cast<half_t>(v[2]),
+                       static_cast<half_t>(v[3])};
+      __builtin_nontemporal_store(q, reinterpret_cast<half4*>(p));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < nv) __builtin_nontemporal_store(static_cast<half_t>(v[i]), p + i);
+  }
+}
+
+// PARAM == kParamF16: scale, min and the output are fp16 and, as in the
+// reference's at::Half instantiation (at::Half operators evaluate in fp32 and
+// round to fp16), the quotient and the sum are each rounded to fp16
+// (quantization_cuda_kernel.cu:182).
+template <int BITS, int SLOTS, int VEC, int PARAM>
 __global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
+  constexpr bool BF16P = PARAM == kParamBF16;
+  constexpr bool F16 = PARAM == kParamF16;
   constexpr int WPT = 8 / BITS;
   constexpr uint32_t FIELD = ((1u << BITS) - 1u) * 0x01010101u;
   const int t = threadIdx.x;
@@ -69,6 +94,9 @@ __global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
   if constexpr (BF16P) {
     sc = bf16_to_f32(static_cast<const uint16_t*>(a.scale)[n]);
     mnv = bf16_to_f32(static_cast<const uint16_t*>(a.mn)[n]);
+  } else if constexpr (F16) {
+    sc = static_cast<float>(static_cast<const half_t*>(a.scale)[n]);
+    mnv = static_cast<float>(static_cast<const half_t*>(a.mn)[n]);
   } else {
     sc = static_cast<const float*>(a.scale)[n];
     mnv = static_cast<const float*>(a.mn)[n];
@@ -81,7 +109,8 @@ __global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
   const float rcp = 1.0f / sc;
   const int shift = static_cast<int>(n & (WPT - 1)) * BITS;
   const uint8_t* grp = a.packed + (n / WPT) * a.G;
-  float* orow = a.out + n * a.G;
+  float* orow = F16 ? nullptr : a.out + n * a.G;
+  half_t* orow_h = F16 ? reinterpret_cast<half_t*>(a.out) + n * a.G : nullptr;
 
   uint32_t w[SLOTS];
 #pragma unroll
@@ -105,15 +134,20 @@ __global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
     float r[4];
     if (__builtin_expect(fast_div, 1)) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) r[i] = exact_quotient(static_cast<float>((f >> (8 * i)) & 0xFFu), sc, rcp) + mnv;
+      for (int i = 0; i < 4; ++i) {
+        const float quo = exact_quotient(static_cast<float>((f >> (8 * i)) & 0xFFu), sc, rcp);
+        r[i] = (F16 ? round_to_half(quo) : quo) + mnv;
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         // quantization_cuda_kernel.cu:182: true division, then add
-        r[i] = static_cast<float>((f >> (8 * i)) & 0xFFu) / sc + mnv;
+        const float quo = static_cast<float>((f >> (8 * i)) & 0xFFu) / sc;
+        r[i] = (F16 ? round_to_half(quo) : quo) + mnv;
       }
     }
-    store_quad<VEC>(orow + 4 * c, min(4, a.G - 4 * c), r);
+    if constexpr (F16) store_quad_half<VEC>(orow_h + 4 * c, min(4, a.G - 4 * c), r);  // rounds the sum to fp16
+    else store_quad<VEC>(orow + 4 * c, min(4, a.G - 4 * c), r);
   }
 }
 
@@ -140,15 +174,15 @@ static UnpackGeometry plan_unpack(int64_t G) {
 
 static bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-template <int BITS, bool BF16P>
+template <int BITS, int PARAM>
 static void launch_unpack_variant(const UnpackArgs& a, bool vec4, dim3 grid, hipStream_t s) {
   if (vec4)
-    hipLaunchKernelGGL((unpack_kernel<BITS, 2, 4, BF16P>), grid, dim3(kBlock), 0, s, a);
+    hipLaunchKernelGGL((unpack_kernel<BITS, 2, 4, PARAM>), grid, dim3(kBlock), 0, s, a);
   else
-    hipLaunchKernelGGL((unpack_kernel<BITS, 2, 1, BF16P>), grid, dim3(kBlock), 0, s, a);
+    hipLaunchKernelGGL((unpack_kernel<BITS, 2, 1, PARAM>), grid, dim3(kBlock), 0, s, a);
 }
 
-template <bool BF16P>
+template <int PARAM>
 static int unpack_common(const uint8_t* packed, int bits, const void* scale, const void* mn,
                          int64_t N, int64_t G, float* out, hipStream_t s) {
   if (bits != 1 && bits != 2 && bits != 4 && bits != 8) return EXACT_E_BITS;
@@ -166,14 +200,14 @@ static int unpack_common(const uint8_t* packed, int bits, const void* scale, con
   a.lpr_log2 = g.lpr_log2;
   a.out = out;
   a.in_vec = (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
-  const bool vec4 = (G % 4 == 0) && aligned(out, 16);
+  const bool vec4 = (G % 4 == 0) && aligned(out, PARAM == kParamF16 ? 8 : 16);
   const int rows_per_wg = kBlock >> g.lpr_log2;
   const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(g.grid_y));
   switch (bits) {
-    case 1: launch_unpack_variant<1, BF16P>(a, vec4, grid, s); break;
-    case 2: launch_unpack_variant<2, BF16P>(a, vec4, grid, s); break;
-    case 4: launch_unpack_variant<4, BF16P>(a, vec4, grid, s); break;
-    default: launch_unpack_variant<8, BF16P>(a, vec4, grid, s); break;
+    case 1: launch_unpack_variant<1, PARAM>(a, vec4, grid, s); break;
+    case 2: launch_unpack_variant<2, PARAM>(a, vec4, grid, s); break;
+    case 4: launch_unpack_variant<4, PARAM>(a, vec4, grid, s); break;
+    default: launch_unpack_variant<8, PARAM>(a, vec4, grid, s); break;
   }
   return launch_status();
 }
@@ -186,12 +220,18 @@ extern "C" {
 
 int exact_unpack_f32(const uint8_t* packed, int bits, const float* scale, const float* mn, int64_t N,
                      int64_t G, float* out, void* stream) {
-  return unpack_common<false>(packed, bits, scale, mn, N, G, out, static_cast<hipStream_t>(stream));
+  return unpack_common<kParamF32>(packed, bits, scale, mn, N, G, out, static_cast<hipStream_t>(stream));
 }
 
 int exact_unpack_bf16param_f32(const uint8_t* packed, int bits, const uint16_t* scale_bf16,
                                const uint16_t* min_bf16, int64_t N, int64_t G, float* out, void* stream) {
-  return unpack_common<true>(packed, bits, scale_bf16, min_bf16, N, G, out, static_cast<hipStream_t>(stream));
+  return unpack_common<kParamBF16>(packed, bits, scale_bf16, min_bf16, N, G, out, static_cast<hipStream_t>(stream));
+}
+
+int exact_unpack_f16(const uint8_t* packed, int bits, const uint16_t* scale_f16, const uint16_t* min_f16,
+                     int64_t N, int64_t G, uint16_t* out_f16, void* stream) {
+  return unpack_common<kParamF16>(packed, bits, scale_f16, min_f16, N, G, reinterpret_cast<float*>(out_f16),
+                                  static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

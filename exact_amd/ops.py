@@ -17,6 +17,7 @@ import math
 
 import torch
 import torch.nn.functional as F
+from torch.amp import custom_bwd, custom_fwd
 from torch.autograd.function import Function
 from torch.utils.weak import WeakIdKeyDictionary
 
@@ -26,7 +27,7 @@ from .cpp_extension import _checks
 from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import quantization as ext_quantization
 from .cpp_extension import spmm
-from .cpp_extension._checks import check_device_tensor, ptr
+from .cpp_extension._checks import FLOAT_OR_HALF, check_device_tensor, ptr
 from .utils import empty_cache, swap_to_cpu
 
 
@@ -84,7 +85,7 @@ def quantize_activation(input, scheme):  # noqa: A002
     _unsupported_modes()
     if scheme:
         scheme.note_use()
-    check_device_tensor(input, "input")
+    check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     bits = config.activation_compression_bits[0]
     packed, scale_bf16, min_bf16 = ext_quantization.minmax_pack(_rows_by_features(input), bits)
     if config.swap:
@@ -107,7 +108,7 @@ def _projection_matrix(D, k, device, dtype):
     if config.rp_matrix_source is not None:
         R = config.rp_matrix_source(D, k, device)
         check_device_tensor(R, "rand_matrix", 2)
-        return R
+        return R.to(dtype)
     if config.rp_distribution == "gaussian":
         return torch.randn((D, k), device=device, dtype=dtype) / k ** 0.5
     # reference ops.py:112-114: Rademacher entries +-1/sqrt(k)
@@ -124,9 +125,12 @@ def kept_columns(width):
 def input2rp(input, kept_acts):  # noqa: A002
     """Reference ops.py:107-118 -> (dim_reduced_input [N, k], rand_matrix [D, k])."""
     assert input.dim() == 2
-    check_device_tensor(input, "input", 2)
+    check_device_tensor(input, "input", 2, FLOAT_OR_HALF)
     N, D = input.shape
     rand_matrix = _projection_matrix(D, kept_acts, input.device, input.dtype).contiguous()
+    if input.dtype != torch.float32:
+        # fp16 activations (autocast): a plain library GEMM, as torch.matmul is in the reference
+        return torch.matmul(input, rand_matrix), rand_matrix
     reduced = torch.empty((N, kept_acts), dtype=input.dtype, device=input.device)
     rc = _lib.lib().exact_rp_fwd_f32(ptr(input), ptr(rand_matrix), N, D, kept_acts, ptr(reduced),
                                      _checks.stream_ptr(input))
@@ -138,8 +142,10 @@ def input2rp(input, kept_acts):  # noqa: A002
 def rp2input(dim_reduced_input, input_shape, rand_matrix):
     """Reference ops.py:121-125."""
     assert dim_reduced_input.dim() == 2
-    check_device_tensor(dim_reduced_input, "dim_reduced_input", 2)
-    check_device_tensor(rand_matrix, "rand_matrix", 2)
+    check_device_tensor(dim_reduced_input, "dim_reduced_input", 2, FLOAT_OR_HALF)
+    check_device_tensor(rand_matrix, "rand_matrix", 2, (dim_reduced_input.dtype,))
+    if dim_reduced_input.dtype != torch.float32:
+        return torch.matmul(dim_reduced_input, rand_matrix.t()).view(input_shape)
     N, k = dim_reduced_input.shape
     D = rand_matrix.shape[0]
     if rand_matrix.shape[1] != k:
@@ -191,10 +197,17 @@ class CompressedActivation:
 # ---------------------------------------------------------------------------
 # autograd Functions
 # ---------------------------------------------------------------------------
+# Inside an autocast region the reference's Functions receive fp16 copies of
+# their floating-point inputs and run with autocast off (custom_fwd(cast_inputs=
+# torch.float16), reference ops.py:130, 260, 313, 377, 408); so do these.
+_amp_fwd = custom_fwd(device_type="cuda", cast_inputs=torch.float16)
+_amp_bwd = custom_bwd(device_type="cuda")
+
 class qlinear(Function):
     """y = x W^T + b, keeping x only in compressed form (reference ops.py:128-178)."""
 
     @staticmethod
+    @_amp_fwd
     def forward(ctx, input, weight, bias=None, quantized=None, randmat=None, scheme=None, rp=True):  # noqa: A002
         if quantized is None:
             kept = CompressedActivation.compress(input, scheme, project=rp)
@@ -205,6 +218,7 @@ class qlinear(Function):
         return F.linear(input, weight, bias)
 
     @staticmethod
+    @_amp_bwd
     def backward(ctx, grad_output):
         kept, ctx.kept = ctx.kept, None
         if kept.randmat is None:
@@ -265,6 +279,7 @@ class qspmm_sum(Function):
     """out = A @ X with sum aggregation (reference ops.py:257-307)."""
 
     @staticmethod
+    @_amp_fwd
     def forward(ctx, row, rowptr, col, value, colptr, csr2csc, has_value, other,
                 quantized=None, randmat=None, scheme=None):
         result = spmm.spmm_sum_fw(row, rowptr, col, value, colptr, csr2csc, other)
@@ -275,6 +290,7 @@ class qspmm_sum(Function):
         return result
 
     @staticmethod
+    @_amp_bwd
     def backward(ctx, grad_outputs):
         row, rowptr, col, value, colptr, csr2csc = ctx.graph
         has_value, value_requires_grad, mat_requires_grad = ctx.flags
@@ -291,6 +307,7 @@ class qspmm_mean(Function):
     """out = D^-1 A @ X, mean aggregation (reference ops.py:310-371)."""
 
     @staticmethod
+    @_amp_fwd
     def forward(ctx, row, rowptr, col, value, rowcount, colptr, csr2csc, has_value, other,
                 quantized=None, randmat=None, scheme=None):
         result = spmm.spmm_mean_fw(row, rowptr, col, value, rowcount, colptr, csr2csc, other)
@@ -301,6 +318,7 @@ class qspmm_mean(Function):
         return result
 
     @staticmethod
+    @_amp_bwd
     def backward(ctx, grad_outputs):
         row, rowptr, col, value, rowcount, colptr, csr2csc = ctx.graph
         has_value, value_requires_grad, mat_requires_grad = ctx.flags
@@ -370,10 +388,12 @@ class qspmm_max(Function):
     """out = max over the entries of each row of val * X[col]  (reference ops.py:374-403)."""
 
     @staticmethod
+    @_amp_fwd
     def forward(ctx, rowptr, col, value, has_value, other, quantized=None, randmat=None, scheme=None):
         return _extreme_forward(ctx, True, rowptr, col, value, has_value, other, quantized, scheme)
 
     @staticmethod
+    @_amp_bwd
     def backward(ctx, grad_outputs):
         return _extreme_backward(ctx, grad_outputs)
 
@@ -382,10 +402,12 @@ class qspmm_min(Function):
     """Reference ops.py:406-436; gradients are routed as for max (spmm.cc:214-241)."""
 
     @staticmethod
+    @_amp_fwd
     def forward(ctx, rowptr, col, value, has_value, other, quantized=None, randmat=None, scheme=None):
         return _extreme_forward(ctx, False, rowptr, col, value, has_value, other, quantized, scheme)
 
     @staticmethod
+    @_amp_bwd
     def backward(ctx, grad_outputs):
         return _extreme_backward(ctx, grad_outputs)
 
@@ -436,7 +458,7 @@ def take_compressed(tensor, project=True):
     if entry is None:
         return None
     version, quantized = entry
-    usable = (config.compress_activation and version == tensor._version
+    usable = (config.compress_activation and version == tensor._version and not torch.is_autocast_enabled()
               and quantized[1] == config.activation_compression_bits[0]
               and not (project and config.kept_frac < 1.0))
     return quantized if usable else None
@@ -447,9 +469,10 @@ def relu_dropout(input, p, for_consumer=False):  # noqa: A002
     result is made in the same pass where the kernel can (2-D rows of a
     multiple of 8 <= 1024 columns, compression on, no projection) and handed
     over to the layer that receives the result."""
-    check_device_tensor(input, "input")
+    check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     bits = None
     if (for_consumer and config.compress_activation and config.kept_frac == 1.0 and input.dim() == 2
+            and input.dtype == torch.float32 and not torch.is_autocast_enabled()
             and ext_quantization.fusable_width(input.shape[1])):
         _unsupported_modes()
         bits = config.activation_compression_bits[0]

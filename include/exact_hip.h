@@ -177,6 +177,40 @@ int exact_relu_dropout_minmax_pack_f32(const float *x, float p, const float *act
                                        float *min_f32, uint16_t *scale_bf16,
                                        uint16_t *min_bf16, void *stream);
 
+/* fp16 activations (row f4: the reference instantiates its kernels for
+ * at::Half as well -- AT_DISPATCH_FLOATING_TYPES_AND_HALF at
+ * quantization_cuda_kernel.cu:132-150, 209-226, 284, 324, 387, 428, 535, 586 --
+ * and its Functions cast their inputs to fp16 under autocast, ops.py:130, 260,
+ * 313).  fp16 tensors are passed as uint16_t bit patterns.  The arithmetic
+ * follows at::Half's operators (evaluate in fp32, round the result to fp16):
+ *   scale = h(h(1 / h(max - min)) * (2^bits - 1));
+ *   q = rn(fmax(h(h(x - min) * scale) + u - 0.5, 0));
+ *   unpacked = h(h(q / scale) + min);
+ * G <= 1024 (the reference's block-size limit). */
+int exact_minmax_pack_f16(const uint16_t *x, const float *noise, uint64_t seed,
+                          uint64_t offset, int64_t N, int64_t G, int bits,
+                          uint8_t *packed, uint16_t *scale_f16, uint16_t *min_f16,
+                          void *stream);
+int exact_unpack_f16(const uint8_t *packed, int bits, const uint16_t *scale_f16,
+                     const uint16_t *min_f16, int64_t N, int64_t G, uint16_t *out_f16,
+                     void *stream);
+/* The mask activations on fp16 tensors: same masks, values rounded to fp16 once
+ * on store (y = h(x * keep * pinv), dx = h(dy / (1 - p)), y = h(x * slope)). */
+int exact_relu_fwd_f16(const uint16_t *x, int64_t n, uint16_t *y, uint32_t *mask, void *stream);
+int exact_relu_bwd_f16(const uint16_t *dy, const uint32_t *mask, int64_t n, uint16_t *dx, void *stream);
+int exact_leaky_relu_fwd_f16(const uint16_t *x, int64_t n, float slope, uint16_t *y,
+                             uint32_t *mask, void *stream);
+int exact_leaky_relu_bwd_f16(const uint16_t *dy, const uint32_t *mask, int64_t n,
+                             float slope, uint16_t *dx, void *stream);
+int exact_dropout_fwd_f16(const uint16_t *x, const float *noise, uint64_t seed,
+                          uint64_t offset, float p, int64_t n, uint16_t *y,
+                          uint32_t *mask, void *stream);
+int exact_relu_dropout_fwd_f16(const uint16_t *x, const float *noise, uint64_t seed,
+                               uint64_t offset, float p, int64_t n, uint16_t *y,
+                               uint32_t *mask, void *stream);
+int exact_dropout_bwd_f16(const uint16_t *dy, const uint32_t *mask, float p,
+                          int64_t n, uint16_t *dx, void *stream);
+
 /* a7. Random projection: out[N, k] = X[N, D] . R[D, k]  (input2rp, ops.py:107-118)
  * and back: out[N, D] = Xr[N, k] . R[D, k]^T  (rp2input, ops.py:121-125).
  * fp32 in, fp32 accumulate on the matrix cores. */

@@ -5,6 +5,7 @@
 // ASan, and compares the results with the C oracle.  Usage:
 //     emu_check [quick|full]
 // `full` adds the benchmark shapes (169343 x 256 and a 169343-node graph).
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -294,6 +295,73 @@ static void check_fused(int64_t N, int64_t G, int bits, bool supplied, std::mt19
   CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "fused scale/min differ N=%ld G=%ld", (long)N, (long)G);
 }
 
+// fp16 entry points against straight loops written here with _Float16 (the
+// Python oracle for them is oracle/exact_oracle_half.py, checked by
+// tests/test_half_kernels.py); supplied noise only.
+static float rh(float x) { return (float)(_Float16)x; }
+
+static void check_half(int64_t N, int64_t G, int bits, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 3.f);
+  std::uniform_real_distribution<float> ud(0.f, 1.f);
+  const int64_t n = N * G, words = (n + 31) / 32;
+  Buf<_Float16> x(n), out(n), y(n), dx(n);
+  Buf<float> u(n);
+  for (int64_t i = 0; i < n; ++i) { x[i] = (_Float16)nd(rng); u[i] = ud(rng); if (u[i] >= 1.f) u[i] = 0.5f; }
+  const int64_t nb = exact_packed_nbytes(N, G, bits);
+  Buf<uint8_t> packed(nb), want(nb);
+  Buf<_Float16> sc(N), mn(N);
+  int rc = exact_minmax_pack_f16((const uint16_t*)x.p, u.p, 1, 2, N, G, bits, packed.p, (uint16_t*)sc.p, (uint16_t*)mn.p, nullptr);
+  CHECK(rc == 0, "pack f16 rc=%d", rc);
+  std::memset(want.p, 0, nb);
+  const int wpt = 8 / bits;
+  int64_t bad = 0;
+  for (int64_t r = 0; r < N; ++r) {
+    float lo = INFINITY, hi = -INFINITY;
+    for (int64_t d = 0; d < G; ++d) { lo = std::fmin(lo, (float)x[r * G + d]); hi = std::fmax(hi, (float)x[r * G + d]); }
+    const float s = rh(rh(1.0f / rh(hi - lo)) * (float)((1 << bits) - 1));
+    bad += ((float)sc[r] != s && !(std::isnan(s) && std::isnan((float)sc[r]))) || (float)mn[r] != lo;
+    for (int64_t d = 0; d < G; ++d) {
+      float t = rh(rh((float)x[r * G + d] - lo) * s);
+      t = t + u[r * G + d];
+      t = t - 0.5f;
+      t = std::fmax(t, 0.f);
+      const int q = (int)std::nearbyint(t);
+      want[(r / wpt) * G + d] |= (uint8_t)(q << ((r % wpt) * bits));
+    }
+  }
+  CHECK(bad == 0, "f16 scale/min differ N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  CHECK(std::memcmp(packed.p, want.p, nb) == 0, "f16 packed differs N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  rc = exact_unpack_f16(packed.p, bits, (const uint16_t*)sc.p, (const uint16_t*)mn.p, N, G, (uint16_t*)out.p, nullptr);
+  bad = 0;
+  for (int64_t r = 0; r < N; ++r)
+    for (int64_t d = 0; d < G; ++d) {
+      const int q = (want[(r / wpt) * G + d] >> ((r % wpt) * bits)) & ((1 << bits) - 1);
+      const _Float16 w = (_Float16)(rh((float)q / (float)sc[r]) + (float)mn[r]);
+      const _Float16 g = out[r * G + d];
+      bad += std::memcmp(&w, &g, 2) != 0 && !(std::isnan((float)w) && std::isnan((float)g));
+    }
+  CHECK(rc == 0 && bad == 0, "f16 unpack differs N=%ld G=%ld bits=%d: %ld", (long)N, (long)G, bits, (long)bad);
+  // masks
+  Buf<uint32_t> m(words);
+  const float p = 0.3f, pinv = (float)(1.0 / (1.0 - (double)p)), p1m = (float)(1.0 - (double)p);
+  rc = exact_relu_dropout_fwd_f16((const uint16_t*)x.p, u.p, 0, 0, p, n, (uint16_t*)y.p, m.p, nullptr);
+  rc |= exact_dropout_bwd_f16((const uint16_t*)x.p, m.p, p, n, (uint16_t*)dx.p, nullptr);
+  bad = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const bool pos = (float)x[i] > 0.f, keep = u[i] > p;
+    const _Float16 wy = (_Float16)(((pos ? (float)x[i] : 0.f) * (keep ? 1.f : 0.f)) * pinv);
+    const _Float16 wdx = (pos && keep) ? (_Float16)((float)x[i] / p1m) : (_Float16)0.f;
+    bad += (float)y[i] != (float)wy || (float)dx[i] != (float)wdx || (((m[i / 32] >> (i % 32)) & 1u) != (uint32_t)(pos && keep));
+  }
+  CHECK(rc == 0 && bad == 0, "f16 relu+dropout differs n=%ld: %ld", (long)n, (long)bad);
+  rc = exact_relu_fwd_f16((const uint16_t*)x.p, n, (uint16_t*)y.p, m.p, nullptr);
+  rc |= exact_leaky_relu_fwd_f16((const uint16_t*)x.p, n, 0.2f, (uint16_t*)y.p, m.p, nullptr);
+  rc |= exact_leaky_relu_bwd_f16((const uint16_t*)x.p, m.p, n, 0.2f, (uint16_t*)dx.p, nullptr);
+  rc |= exact_relu_bwd_f16((const uint16_t*)x.p, m.p, n, (uint16_t*)dx.p, nullptr);
+  rc |= exact_dropout_fwd_f16((const uint16_t*)x.p, nullptr, 3, 4, p, n, (uint16_t*)y.p, m.p, nullptr);
+  CHECK(rc == 0, "f16 mask entry points rc=%d", rc);
+}
+
 int main(int argc, char** argv) {
   std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
@@ -333,6 +401,10 @@ int main(int argc, char** argv) {
     for (int bits : {1, 2, 4, 8})
       for (int supplied = 0; supplied < 2; ++supplied) check_fused(f[0], f[1], bits, supplied, rng);
   std::printf("fused epilogues ok (failures so far %d)\n", g_fail);
+  const int64_t hs[][2] = {{1, 1}, {5, 3}, {37, 25}, {64, 32}, {33, 40}, {203, 256}, {61, 602}, {16, 1024}, {19, 520}, {8, 8}};
+  for (auto& f : hs)
+    for (int bits : {1, 2, 4, 8}) check_half(f[0], f[1], bits, rng);
+  std::printf("fp16 entry points ok (failures so far %d)\n", g_fail);
   if (mode == "full") {
     for (int bits : {1, 2, 4, 8}) check_quant(169343, 256, bits, bits == 2, rng);
     std::printf("full-size quant ok (failures so far %d)\n", g_fail);

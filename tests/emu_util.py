@@ -246,3 +246,70 @@ def relu_dropout_minmax_pack(x, prob, bits, act_noise=None, noise=None, act_seed
         return None
     assert (packed[nb:] == 0xA5).all() and (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
     return y[:n].reshape(N, G), mask[:words], packed[:nb], s32, m32, sbf, mbf
+
+
+# ---- fp16 entry points -------------------------------------------------------
+def f16(a):
+    return np.ascontiguousarray(a, dtype=np.float16)
+
+
+def minmax_pack_f16(x, bits, noise=None, seed=0, offset=0, guard=64, expect_rc=0):
+    x = f16(x)
+    N, G = x.shape
+    nb = int(emu().exact_packed_nbytes(N, G, bits))
+    packed = np.full(nb + guard, 0xA5, np.uint8)
+    sc, mn = np.zeros(N, np.float16), np.zeros(N, np.float16)
+    noise = None if noise is None else f32(noise)
+    rc = emu().exact_minmax_pack_f16(p(x), p(noise), seed, offset, N, G, bits, p(packed), p(sc), p(mn), None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (packed[nb:] == 0xA5).all()
+    return packed[:nb], sc, mn
+
+
+def unpack_f16(packed, bits, scale, mn, N, G, guard=64):
+    out = np.full(N * G + guard, np.float16(-123.0), np.float16)
+    rc = emu().exact_unpack_f16(p(np.ascontiguousarray(packed)), bits, p(f16(scale)), p(f16(mn)), N, G, p(out), None)
+    assert rc == 0, rc
+    assert (out[N * G:] == np.float16(-123.0)).all()
+    return out[:N * G].reshape(N, G)
+
+
+def _mask_fwd_f16(fn, x, *args, guard=8):
+    x = f16(x).reshape(-1)
+    n = x.size
+    y = np.full(n + guard, np.float16(7.0), np.float16)
+    words = (n + 31) // 32
+    mask = np.full(words + guard, 0x5A5A5A5A, np.uint32)
+    assert fn(x, n, y, mask, *args) == 0
+    assert (y[n:] == 7.0).all() and (mask[words:] == 0x5A5A5A5A).all()
+    return y[:n], mask[:words]
+
+
+def relu_fwd_f16(x):
+    return _mask_fwd_f16(lambda x, n, y, m: emu().exact_relu_fwd_f16(p(x), n, p(y), p(m), None), x)
+
+
+def leaky_relu_fwd_f16(x, slope):
+    return _mask_fwd_f16(lambda x, n, y, m: emu().exact_leaky_relu_fwd_f16(p(x), n, slope, p(y), p(m), None), x)
+
+
+def dropout_fwd_f16(x, prob, noise=None, seed=0, offset=0, relu=False):
+    noise = None if noise is None else f32(noise).reshape(-1)
+    fn = emu().exact_relu_dropout_fwd_f16 if relu else emu().exact_dropout_fwd_f16
+    return _mask_fwd_f16(lambda x, n, y, m: fn(p(x), p(noise), seed, offset, prob, n, p(y), p(m), None), x)
+
+
+def mask_bwd_f16(kind, dy, mask, arg=None):
+    dy = f16(dy).reshape(-1)
+    dx = np.zeros_like(dy)
+    mask = np.ascontiguousarray(mask, np.uint32)
+    if kind == "relu":
+        rc = emu().exact_relu_bwd_f16(p(dy), p(mask), dy.size, p(dx), None)
+    elif kind == "leaky":
+        rc = emu().exact_leaky_relu_bwd_f16(p(dy), p(mask), dy.size, arg, p(dx), None)
+    else:
+        rc = emu().exact_dropout_bwd_f16(p(dy), p(mask), arg, dy.size, p(dx), None)
+    assert rc == 0, rc
+    return dx

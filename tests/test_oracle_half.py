@@ -1,0 +1,95 @@
+"""Pins oracle/exact_oracle_half.py against torch's CPU fp16 tensor arithmetic
+(every torch op on an fp16 CPU tensor evaluates in fp32 and rounds to fp16, the
+behaviour of at::Half's operators that the reference's fp16 kernels rely on)."""
+import numpy as np
+import pytest
+import torch
+
+import exact_oracle as o
+import exact_oracle_half as oh
+
+F16, F32 = np.float16, np.float32
+
+
+def rows(N, G, seed, spread=3.0):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((N, G)) * spread).astype(F16)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_scale_matches_torch_half_arithmetic(bits):
+    x = torch.from_numpy(rows(300, 40, bits))
+    mn, mx = x.min(1).values, x.max(1).values
+    want = (2 ** bits - 1) / (mx - mn)              # reciprocal() * int on an fp16 tensor, as ops.py:39 does
+    got = oh.compute_scale(mn.float().numpy(), mx.float().numpy(), bits)
+    assert want.dtype == torch.float16 and np.array_equal(got.astype(F16).view(np.uint16), want.numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_quantised_values_match_torch_half_arithmetic(bits):
+    xn = rows(257, 24, 10 + bits)
+    xn[3] = xn[3, 0]                                  # constant row
+    noise = np.random.default_rng(bits).random(xn.shape, dtype=F32)
+    x = torch.from_numpy(xn)
+    mn, mx = x.min(1).values, x.max(1).values
+    scale = (2 ** bits - 1) / (mx - mn)
+    t = (x - mn[:, None]) * scale[:, None]            # two fp16 roundings
+    t = t.float() + torch.from_numpy(noise) - 0.5     # Half + float -> float
+    q = torch.clamp(torch.nan_to_num(t, nan=0.0), min=0).round().to(torch.int64).numpy()
+    packed, sc, m = oh.quantize_activation(xn, bits, noise)
+    assert np.array_equal(sc.view(np.uint16), scale.numpy().view(np.uint16)) and np.array_equal(m, mn.numpy())
+    # unpack the oracle's bytes with the fp32 oracle's layout code and compare the codes
+    wpt = 8 // bits
+    N, G = xn.shape
+    n_round = N + (wpt - N % wpt) % wpt
+    p = packed[:(n_round // wpt) * G].reshape(n_round // wpt, 1, G).astype(np.int64)
+    codes = ((p >> (np.arange(wpt) * bits).reshape(1, wpt, 1)) & (2 ** bits - 1)).reshape(n_round, G)[:N]
+    keep = q <= 2 ** bits - 1                          # a spill into the next field is not a code of its own
+    assert np.array_equal(codes[keep], q[keep]) and keep.mean() > 0.999
+    assert packed.size == o.packed_nbytes(N, G, bits) and packed[-1] == 0
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+def test_unpack_matches_torch_half_arithmetic(bits):
+    xn = rows(130, 16, 20 + bits)
+    noise = np.full(xn.shape, 0.5, F32)
+    packed, sc, mn = oh.quantize_activation(xn, bits, noise)
+    out = oh.unpack(packed, bits, sc, mn, *xn.shape)
+    wpt = 8 // bits
+    N, G = xn.shape
+    n_round = N + (wpt - N % wpt) % wpt
+    p = packed[:(n_round // wpt) * G].reshape(n_round // wpt, 1, G).astype(np.int64)
+    codes = ((p >> (np.arange(wpt) * bits).reshape(1, wpt, 1)) & (2 ** bits - 1)).reshape(n_round, G)[:N]
+    q = torch.from_numpy(codes).to(torch.float16)
+    want = q / torch.from_numpy(sc)[:, None] + torch.from_numpy(mn)[:, None]
+    assert out.dtype == F16 and np.array_equal(out.view(np.uint16), want.numpy().view(np.uint16))
+    # and the round trip stays within one quantisation step (+ fp16 rounding of the result)
+    step = 1.0 / sc.astype(F32)
+    err = np.abs(out.astype(F32) - xn.astype(F32))
+    ok = np.isfinite(step)
+    assert (err[ok] <= (step[ok, None] * 1.0 + np.abs(xn[ok].astype(F32)) * 2e-3 + 1e-3)).all()
+
+
+def test_mask_ops_match_torch_half():
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(1000) * 4).astype(F16)
+    g = (rng.standard_normal(1000) * 4).astype(F16)
+    u = rng.random(1000, dtype=F32)
+    xt, gt = torch.from_numpy(x), torch.from_numpy(g)
+    y, m = oh.relu_fwd(x)
+    assert np.array_equal(y, torch.relu(xt).numpy()) and np.array_equal(oh.relu_bwd(g, m), torch.where(xt > 0, gt, torch.zeros_like(gt)).numpy())
+    y, m = oh.leaky_relu_fwd(x, 0.2)
+    want = torch.where(xt > 0, xt, (xt.float() * 0.2).half())
+    assert np.array_equal(y.view(np.uint16), want.numpy().view(np.uint16))
+    keep = torch.from_numpy(u) > 0.3
+    pinv = np.float32(1.0 / (1.0 - float(np.float32(0.3))))
+    want = (xt.float() * keep.float() * float(pinv)).half()
+    y, m = oh.dropout_fwd(x, 0.3, u)
+    assert np.array_equal(y.view(np.uint16), want.numpy().view(np.uint16)) and np.array_equal(m, o._pack_bits(keep.numpy()))
+    p1m = np.float32(1.0 - float(np.float32(0.3)))
+    want = torch.where(keep, (gt.float() / float(p1m)).half(), torch.zeros_like(gt))
+    assert np.array_equal(oh.dropout_bwd(g, m, 0.3).view(np.uint16), want.numpy().view(np.uint16))
+    y2, m2 = oh.dropout_fwd(x, 0.3, u, relu=True)
+    y1, m1 = oh.relu_fwd(x)
+    y3, m3 = oh.dropout_fwd(y1, 0.3, u)
+    assert np.array_equal(y2.view(np.uint16), y3.view(np.uint16)) and np.array_equal(m2, m1 & m3)
