@@ -222,6 +222,8 @@ int exact_spmm_csr_f32(const void* rowptr, const void* col, const float* val, in
   if (reduce != EXACT_REDUCE_SUM && reduce != EXACT_REDUCE_MEAN) return EXACT_E_ARG;
   if (M < 0 || K < 0 || nnz < 0 || n_cols < 0 || n_cols > 0x7FFFFFFFll) return EXACT_E_SHAPE;
   if (idx_bytes == 4 && nnz > 0x7FFFFFFFll) return EXACT_E_SHAPE;
+  // launch-grid limits: 2^31 - 1 workgroups of 256 rows (pre-pass) resp. 256 entries (main kernel)
+  if (M > (int64_t{1} << 38) || nnz > (int64_t{1} << 38) || K > (int64_t{1} << 24)) return EXACT_E_SHAPE;
   if (M == 0 || K == 0) return EXACT_OK;
   if (!rowptr || !out || (nnz > 0 && (!col || !X))) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -128,6 +128,7 @@ int exact_spmm_csr_minmax_f32(const void* rowptr, const void* col, const float* 
   if (idx_bytes != 4 && idx_bytes != 8) return EXACT_E_ARG;
   if (M < 0 || K < 0 || nnz < 0 || n_cols < 0 || n_cols > 0x7FFFFFFFll) return EXACT_E_SHAPE;
   if (idx_bytes == 4 && nnz > 0x7FFFFFFFll) return EXACT_E_SHAPE;
+  if (M > (int64_t{1} << 32) || K > (int64_t{1} << 24)) return EXACT_E_SHAPE;  // launch-grid limits
   if (M == 0 || K == 0) return EXACT_OK;
   if (!rowptr || !out || !arg_out || (nnz > 0 && (!col || !X))) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -147,7 +148,7 @@ int exact_sddmm_f32(const void* row, const void* rowptr, const void* col, int id
                     const float* grad, int64_t nnz, int64_t K, int reduce, float* out, void* stream) {
   if (idx_bytes != 4 && idx_bytes != 8) return EXACT_E_ARG;
   if (reduce != EXACT_REDUCE_SUM && reduce != EXACT_REDUCE_MEAN) return EXACT_E_ARG;
-  if (nnz < 0 || K < 0) return EXACT_E_SHAPE;
+  if (nnz < 0 || K < 0 || nnz > (int64_t{1} << 32)) return EXACT_E_SHAPE;  // one wavefront per entry, 4 per workgroup
   if (nnz == 0) return EXACT_OK;
   if (!row || !rowptr || !col || !mat || !grad || !out) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -3,8 +3,10 @@
 // Calls every C-ABI entry point on heap buffers of EXACTLY the documented
 // sizes, so that any out-of-bounds load or store of a kernel is reported by
 // ASan, and compares the results with the C oracle.  Usage:
-//     emu_check [quick|full]
-// `full` adds the benchmark shapes (169343 x 256 and a 169343-node graph).
+//     emu_check [quick|large|full]
+// `large` adds grids of thousands of workgroups (20011 x 256, a 20000-node
+// graph; minutes); `full` adds the benchmark shapes (169343 x 256 and a
+// 169343-node graph; hours under the sanitizer).
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -405,6 +407,19 @@ int main(int argc, char** argv) {
   for (auto& f : hs)
     for (int bits : {1, 2, 4, 8}) check_half(f[0], f[1], bits, rng);
   std::printf("fp16 entry points ok (failures so far %d)\n", g_fail);
+  if (mode == "large" || mode == "full") {
+    for (int bits : {1, 2, 4, 8}) check_quant(20011, 256, bits, bits == 4, rng);
+    check_quant(3001, 1024, 2, false, rng);
+    check_masks(20011ll * 256 + 3, rng);
+    check_spmm(20000, 20000, 256, 14, 5000, rng);
+    check_spmm(20000, 20000, 100, 14, 5000, rng);
+    check_extra(5000, 5000, 64, 10, rng);
+    check_rp(20011, 256, 32, rng);
+    check_rp(5003, 602, 76, rng);
+    check_fused(20011, 256, 2, false, rng);
+    check_half(20011, 256, 2, rng);
+    std::printf("large shapes ok (failures so far %d)\n", g_fail);
+  }
   if (mode == "full") {
     for (int bits : {1, 2, 4, 8}) check_quant(169343, 256, bits, bits == 2, rng);
     std::printf("full-size quant ok (failures so far %d)\n", g_fail);
