@@ -124,7 +124,11 @@ def test_gcn_step_in_fp16(backend):
 @pytest.mark.gpu
 def test_training_step_under_autocast(cuda):
     """torch.autocast: the Functions cast their inputs to fp16 (custom_fwd), the
-    kept activations are the fp16 ones, parameters and their gradients stay fp32."""
+    kept activations are the fp16 ones, parameters and their gradients stay fp32
+    (the bias additions promote the layer outputs back to fp32)."""
+    seen = []
+    real = extq.minmax_pack
+    import unittest.mock as mock
     _, adj = graph(500, 4000, 3, cuda)
     torch.manual_seed(2)
     model = exact.QModule(GCN(32, 64, 5, 3, dropout=0.5, batch_norm=True)).to(cuda).train()
@@ -132,15 +136,16 @@ def test_training_step_under_autocast(cuda):
     labels = torch.randint(0, 5, (500,), device=cuda)
     opt = torch.optim.Adam(model.parameters(), lr=0.01)
     losses = []
-    for _ in range(5):
-        opt.zero_grad()
-        with torch.autocast("cuda", dtype=torch.float16):
-            out = model(x, adj)
-            loss = F.cross_entropy(out.float(), labels)
-        loss.backward()
-        opt.step()
-        losses.append(loss.item())
-    assert out.dtype == torch.float16
+    with mock.patch.object(extq, "minmax_pack", lambda data, bits, want_fp32=False: seen.append(data.dtype) or real(data, bits, want_fp32)):
+        for _ in range(5):
+            opt.zero_grad()
+            with torch.autocast("cuda", dtype=torch.float16):
+                out = model(x, adj)
+                loss = F.cross_entropy(out.float(), labels)
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+    assert torch.float16 in seen                     # the linear layers compressed fp16 copies of their inputs
     assert all(np.isfinite(l) for l in losses)
     assert all(p.grad is not None and p.grad.dtype == torch.float32 and torch.isfinite(p.grad).all()
                for p in model.parameters())
