@@ -113,7 +113,7 @@ __device__ __forceinline__ uint16_t half_bits(float x) {
 // Steps: quad_perm [1,0,3,2] and [2,3,0,1] fold a quad, after which the four
 // lanes of a quad agree, so the half-row mirror (lane i <-> 7 - i) delivers "the
 // other quad"; row_ror:8 delivers the other half of a 16-lane row; lanes 16
-// apart swap through ds_swizzle, lanes 32 apart through ds_bpermute.
+// and 32 apart (rows spread over more than one DPP row) go through ds_bpermute.
 __device__ __forceinline__ int order_key(float f) {
   const int b = __float_as_int(f);
   return b ^ ((b >> 31) & 0x7FFFFFFF);
@@ -143,14 +143,9 @@ __device__ __forceinline__ void group_minmax(float& mn, float& mx, int span) {
     lo = min(lo, dpp_lanes<0x128>(lo));
     hi = max(hi, dpp_lanes<0x128>(hi));
   }
-  if (span >= 32) {
-    constexpr int kSwap16 = 0x401F;  // bit-mask mode: and 0x1F, or 0, xor 0x10
-    lo = min(lo, __builtin_amdgcn_ds_swizzle(lo, kSwap16));
-    hi = max(hi, __builtin_amdgcn_ds_swizzle(hi, kSwap16));
-  }
-  if (span >= 64) {
-    lo = min(lo, __shfl_xor(lo, 32));
-    hi = max(hi, __shfl_xor(hi, 32));
+  for (int m = 16; m < span; m <<= 1) {
+    lo = min(lo, __shfl_xor(lo, m));
+    hi = max(hi, __shfl_xor(hi, m));
   }
   mn = key_value(lo);
   mx = key_value(hi);

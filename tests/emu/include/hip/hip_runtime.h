@@ -350,22 +350,6 @@ inline int update_dpp_i32(int v, int ctrl, int row_mask, int bank_mask, bool bou
 inline float update_dpp_any(float v, int c, int rm, int bm, bool bc) { return update_dpp_f32(v, c, rm, bm, bc); }
 inline int update_dpp_any(int v, int c, int rm, int bm, bool bc) { return update_dpp_i32(v, c, rm, bm, bc); }
 
-// ds_swizzle in bit-mask mode (offset bit 15 clear): within each group of 32
-// lanes, lane l reads lane ((l & and) | or) ^ xor; an inactive source reads 0.
-inline int ds_swizzle(int v, int pattern) {
-  WaveState* w;
-  int lane;
-  const int buf = wave_collect(static_cast<uint32_t>(v), w, lane);
-  if (pattern & 0x8000) {
-    std::fprintf(stderr, "hip emulator: unsupported swizzle mode 0x%x\n", pattern);
-    std::abort();
-  }
-  const int a = pattern & 31, o = (pattern >> 5) & 31, x = (pattern >> 10) & 31;
-  const int src = (lane & ~31) | ((((lane & 31) & a) | o) ^ x);
-  if (!((w->mask[buf] >> src) & 1)) return 0;
-  return static_cast<int>(static_cast<uint32_t>(w->slot[buf][src]));
-}
-
 // v_bitop3_b32: bit i of the result = truth table bit ((a_i << 2) | (b_i << 1) | c_i)
 inline uint32_t bitop3(uint32_t a, uint32_t b, uint32_t c, int table) {
   uint32_t out = 0;
@@ -462,7 +446,6 @@ static inline uint64_t __ballot(bool p) { return hipemu::ballot(p); }
 #define __builtin_amdgcn_readfirstlane(v) static_cast<int>(hipemu::readfirstlane_u32(static_cast<uint32_t>(v)))
 #define __builtin_amdgcn_mov_dpp(v, ctrl, rm, bm, bc) hipemu::mov_dpp((v), (ctrl), (rm), (bm), (bc))
 #define __builtin_amdgcn_update_dpp(old, v, ctrl, rm, bm, bc) hipemu::update_dpp_any((v), (ctrl), (rm), (bm), (bc))
-#define __builtin_amdgcn_ds_swizzle(v, pattern) hipemu::ds_swizzle((v), (pattern))
 #define __builtin_amdgcn_bitop3_b32(a, b, c, table) hipemu::bitop3((a), (b), (c), (table))
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) hipemu::mfma_f32_32x32x2f32((a), (b), (c), (x), (y), (z))
 
