@@ -15,14 +15,14 @@ from . import cpp_extension, ops, spmm  # noqa: F401
 from .conf import config  # noqa: F401
 from .gatconv import QCustomGATConv  # noqa: F401
 from .layers import (QELU, QMLP, QBatchNorm1d, QDropout, QDropout2, QGCN2Conv, QGCNConv,  # noqa: F401
-                     QGraphConv, QLeakyReLU, QLinear, QReLU, QReLUDropout, QSAGEConv)
+                     QGENConv, QGraphConv, QLeakyReLU, QLinear, QReLU, QReLUDropout, QSAGEConv)
 from .module import QModule  # noqa: F401
 from .sparse import SparseTensor, gcn_norm  # noqa: F401
 from .utils import (cast_adj, cast_low_bit_int, compute_tensor_bytes,  # noqa: F401
                     exp_recorder, get_memory_usage)
 
 __all__ = ["config", "QModule", "QLinear", "QGCNConv", "QSAGEConv", "QBatchNorm1d", "QReLU", "QDropout",
-           "QDropout2", "QLeakyReLU", "QELU", "QReLUDropout", "QGCN2Conv", "QGraphConv", "QMLP", "QCustomGATConv", "SparseTensor", "gcn_norm", "ops", "spmm", "cpp_extension", "install_as_exact"]
+           "QDropout2", "QLeakyReLU", "QELU", "QReLUDropout", "QGCN2Conv", "QGENConv", "QGraphConv", "QMLP", "QCustomGATConv", "SparseTensor", "gcn_norm", "ops", "spmm", "cpp_extension", "install_as_exact"]
 
 
 def install_as_exact():

@@ -8,7 +8,7 @@ from torch.nn import Parameter
 
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
-from .nn import GCN2Conv, GCNConv, GraphConv, SAGEConv, glorot
+from .nn import GCN2Conv, GCNConv, GENConv, GraphConv, SAGEConv, glorot
 from .ops import input2rp, qbatch_norm, qelu, qlinear, quantize_activation, relu_dropout, take_compressed
 from .qsheme import QScheme
 from .spmm import QMatmul, qmatmul
@@ -159,6 +159,17 @@ class QMLP(torch.nn.Sequential):
                 blocks.append(QReLU())
                 blocks.append(QDropout(dropout))
         super().__init__(*blocks)
+
+
+class QGENConv(GENConv):
+    """layers.py:50-63: the MLP is a QMLP and the message ReLU keeps a 1-bit mask."""
+
+    def _make_mlp(self, channels, norm):
+        return QMLP(channels, norm)
+
+    def message(self, x_j, edge_attr=None):
+        msg = x_j if edge_attr is None else x_j + edge_attr
+        return ext_quantization.act_quantized_relu(msg) + self.eps
 
 
 class QReLU(torch.nn.Module):

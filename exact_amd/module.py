@@ -1,7 +1,7 @@
 """QModule: wrap a model and swap its stock layers for the quantised ones, as
 exact/exact/module.py:18-112 of the reference does for the layer types on this
 library's path (Linear, BatchNorm1d, ReLU, Dropout, GCNConv, SAGEConv, GCN2Conv,
-GraphConv, CustomGATConv; GENConv is not provided)."""
+GraphConv, CustomGATConv, GENConv)."""
 from collections import OrderedDict
 
 import torch
@@ -9,12 +9,12 @@ import torch.nn as nn
 
 from .conf import config
 from .gatconv import QCustomGATConv
-from .layers import (QBatchNorm1d, QDropout, QDropout2, QGCN2Conv, QGCNConv, QGraphConv, QLinear, QReLU,
-                     QReLUDropout, QSAGEConv)
-from .nn import CustomGATConv, GCN2Conv, GCNConv, GraphConv, ReLUDropout, SAGEConv
+from .layers import (QBatchNorm1d, QDropout, QDropout2, QGCN2Conv, QGCNConv, QGENConv, QGraphConv, QLinear,
+                     QReLU, QReLUDropout, QSAGEConv)
+from .nn import CustomGATConv, GCN2Conv, GCNConv, GENConv, GraphConv, ReLUDropout, SAGEConv
 
 _QUANTIZED = (QBatchNorm1d, QLinear, QReLU, QGCNConv, QDropout, QDropout2, QSAGEConv, QReLUDropout, QGCN2Conv,
-              QGraphConv, QCustomGATConv)
+              QGraphConv, QCustomGATConv, QGENConv)
 
 
 def _is_pyg(child, name):
@@ -63,6 +63,18 @@ class QModule(nn.Module):
                 new = QCustomGATConv(child.in_channels, child.out_channels, child.heads, child.concat,
                                      child.negative_slope, child.dropout, child.add_self_loops,
                                      child.bias is not None, child.residual, child.use_attn_dst)
+            elif isinstance(child, GENConv):
+                norm = "batch"
+                for m in child.mlp:
+                    if isinstance(m, nn.LayerNorm):
+                        norm = "layer"
+                    elif isinstance(m, nn.InstanceNorm1d):
+                        norm = "instance"
+                new = QGENConv(child.in_channels, child.out_channels, child.aggr, child.initial_t,
+                               child.aggr == "softmax" and isinstance(child.t, nn.Parameter), child.initial_p,
+                               isinstance(child.p, nn.Parameter), child.msg_norm is not None,
+                               child.msg_norm is not None and child.msg_norm.scale.requires_grad, norm,
+                               sum(isinstance(m, nn.Linear) for m in child.mlp), child.eps)
             else:
                 QModule.convert_layers(child)
                 continue

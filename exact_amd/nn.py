@@ -225,15 +225,16 @@ class GCN2Conv(torch.nn.Module):
         return self._addmm(x, x, self.weight1) + self._addmm(x_0, x_0, self.weight2)
 
 
-def edge_softmax(score, row, num_rows):
+def edge_softmax(score, row, num_rows, eps=1e-16):
     """Softmax of score[E, H] over the entries that share a row (PyG's
-    utils.softmax: shift by the group maximum, + 1e-16 in the denominator)."""
+    utils.softmax: shift by the group maximum, + 1e-16 in the denominator;
+    torch_scatter's scatter_softmax is the same with eps = 0)."""
     idx = row.view(-1, 1).expand_as(score)
     top = torch.full((num_rows, score.size(1)), float("-inf"), dtype=score.dtype, device=score.device)
     top = top.scatter_reduce(0, idx, score.detach(), "amax", include_self=True)
     e = (score - top.index_select(0, row)).exp()
     denom = torch.zeros((num_rows, score.size(1)), dtype=score.dtype, device=score.device).index_add_(0, row, e)
-    return e / (denom.index_select(0, row) + 1e-16)
+    return e / (denom.index_select(0, row) + eps)
 
 
 class CustomGATConv(torch.nn.Module):
@@ -328,3 +329,105 @@ class CustomGATConv(torch.nn.Module):
         if self.bias is not None:
             out = out + self.bias
         return out
+
+
+class MLP(torch.nn.Sequential):
+    """Linear (-> norm) -> ReLU -> Dropout blocks, the MLP of PyG's GENConv."""
+
+    def __init__(self, channels, norm=None, bias=True, dropout=0.0):
+        blocks = []
+        for i in range(1, len(channels)):
+            blocks.append(Linear(channels[i - 1], channels[i], bias))
+            if i < len(channels) - 1:
+                if norm == "batch":
+                    blocks.append(torch.nn.BatchNorm1d(channels[i], affine=True))
+                elif norm == "layer":
+                    blocks.append(torch.nn.LayerNorm(channels[i], elementwise_affine=True))
+                elif norm == "instance":
+                    blocks.append(torch.nn.InstanceNorm1d(channels[i], affine=False))
+                elif norm:
+                    raise NotImplementedError(f'Normalization layer "{norm}" not supported.')
+                blocks.append(torch.nn.ReLU())
+                blocks.append(torch.nn.Dropout(dropout))
+        super().__init__(*blocks)
+
+
+class MessageNorm(torch.nn.Module):
+    """msg / |msg| * |x| * scale (PyG's MessageNorm)."""
+
+    def __init__(self, learn_scale=False):
+        super().__init__()
+        self.scale = Parameter(torch.Tensor([1.0]), requires_grad=learn_scale)
+
+    def reset_parameters(self):
+        self.scale.data.fill_(1.0)
+
+    def forward(self, x, msg, p=2):
+        return F.normalize(msg, p=p, dim=-1) * x.norm(p=p, dim=-1, keepdim=True) * self.scale
+
+
+class GENConv(torch.nn.Module):
+    """The generalised aggregation layer of DeeperGCN that the reference's
+    QGENConv subclasses (layers.py:50-63; PyG 1.7 GENConv): per edge the
+    message relu(x_j) + eps, aggregated per target node with a softmax (optionally
+    stop-gradient) or a power mean, added to x_i and passed through an MLP.
+    Entry (i, j) of adj_t carries the message from j to i; edge features are
+    not supported on this path."""
+
+    def __init__(self, in_channels, out_channels, aggr="softmax", t=1.0, learn_t=False, p=1.0, learn_p=False,
+                 msg_norm=False, learn_msg_scale=False, norm="batch", num_layers=2, eps=1e-7):
+        super().__init__()
+        assert aggr in ("softmax", "softmax_sg", "power")
+        self.in_channels, self.out_channels, self.aggr, self.eps = in_channels, out_channels, aggr, eps
+        channels = [in_channels] + [in_channels * 2] * (num_layers - 1) + [out_channels]
+        self.mlp = self._make_mlp(channels, norm)
+        self.msg_norm = MessageNorm(learn_msg_scale) if msg_norm else None
+        self.initial_t, self.initial_p = t, p
+        self.t = Parameter(torch.Tensor([t]), requires_grad=True) if (learn_t and aggr == "softmax") else t
+        self.p = Parameter(torch.Tensor([p]), requires_grad=True) if learn_p else p
+
+    def _make_mlp(self, channels, norm):
+        return MLP(channels, norm=norm)
+
+    def reset_parameters(self):
+        for m in self.mlp:
+            if hasattr(m, "reset_parameters"):
+                m.reset_parameters()
+        if self.msg_norm is not None:
+            self.msg_norm.reset_parameters()
+        if isinstance(self.t, Parameter):
+            self.t.data.fill_(self.initial_t)
+        if isinstance(self.p, Parameter):
+            self.p.data.fill_(self.initial_p)
+
+    def message(self, x_j, edge_attr=None):
+        msg = x_j if edge_attr is None else x_j + edge_attr
+        return F.relu(msg) + self.eps
+
+    def aggregate(self, inputs, row, num_rows):
+        if self.aggr in ("softmax", "softmax_sg"):
+            alpha = edge_softmax(inputs * self.t, row, num_rows, eps=0.0)
+            if self.aggr == "softmax_sg":
+                alpha = alpha.detach()
+            out = torch.zeros((num_rows, inputs.size(1)), dtype=inputs.dtype, device=inputs.device)
+            return out.index_add_(0, row, inputs * alpha)
+        lo, hi = 1e-7, 1e1
+        powered = torch.pow(inputs.clamp(lo, hi), self.p)
+        total = torch.zeros((num_rows, inputs.size(1)), dtype=inputs.dtype, device=inputs.device).index_add_(0, row, powered)
+        count = torch.zeros(num_rows, dtype=inputs.dtype, device=inputs.device).index_add_(
+            0, row, torch.ones_like(row, dtype=inputs.dtype)).clamp_(min=1)
+        return torch.pow((total / count.unsqueeze(-1)).clamp(lo, hi), 1 / self.p)
+
+    def forward(self, x, edge_index, edge_attr=None, size=None):
+        if edge_attr is not None:
+            raise NotImplementedError("edge features are not supported on the SparseTensor path")
+        if isinstance(x, torch.Tensor):
+            x = (x, x)
+        row, col, _ = edge_index.coo()
+        row, col = row.long(), col.long()
+        out = self.aggregate(self.message(x[0].index_select(0, col)), row, edge_index.sparse_size(0))
+        if self.msg_norm is not None:
+            out = self.msg_norm(x[0], out)
+        if x[1] is not None:
+            out = out + x[1]
+        return self.mlp(out)

@@ -36,7 +36,7 @@ def copy_params(dst, src):
 
 def grads_of(layer, out):
     out.square().sum().backward()
-    return {k: p.grad.detach().clone() for k, p in layer.named_parameters()}
+    return {k: p.grad.detach().clone() for k, p in layer.named_parameters() if p.grad is not None}
 
 
 def close(a, b, backend, loose=False):
@@ -163,3 +163,52 @@ def test_qmlp_block(backend):
     close(mlp(x), want, backend)
     with pytest.raises(NotImplementedError):
         exact.QMLP([4, 4, 4], "layer")
+
+
+def dense_gen(layer, A, x):
+    """Dense restatement of GENConv's aggregation."""
+    M = torch.from_numpy(A.toarray() != 0).to(x.device)                  # [i, j]
+    msg = F.relu(x) + layer.eps                                           # [j, C]
+    if layer.aggr in ("softmax", "softmax_sg"):
+        score = (msg * layer.t).unsqueeze(0).expand(M.shape[0], -1, -1).masked_fill(~M.unsqueeze(-1), float("-inf"))
+        alpha = torch.softmax(score, dim=1)
+        alpha = torch.nan_to_num(alpha, nan=0.0)                          # rows without neighbours
+        agg = (alpha * msg.unsqueeze(0)).sum(1)
+    else:
+        powered = msg.clamp(1e-7, 1e1).pow(layer.p)
+        cnt = M.sum(1, keepdim=True).clamp(min=1)
+        agg = ((M.unsqueeze(-1) * powered.unsqueeze(0)).sum(1) / cnt).clamp(1e-7, 1e1).pow(1 / layer.p)
+    if layer.msg_norm is not None:
+        agg = F.normalize(agg, p=2, dim=-1) * x.norm(p=2, dim=-1, keepdim=True) * layer.msg_norm.scale
+    return layer.mlp(agg + x)
+
+
+@pytest.mark.parametrize("aggr,msg_norm,learn", [("softmax", False, True), ("softmax_sg", True, False), ("power", False, True)])
+def test_gen_conv(backend, aggr, msg_norm, learn):
+    A, adj = graph(50, 260, 4, backend)
+    torch.manual_seed(5)
+    stock = xnn.GENConv(12, 8, aggr=aggr, t=0.7, learn_t=learn, p=2.0, learn_p=learn, msg_norm=msg_norm,
+                        learn_msg_scale=msg_norm, num_layers=2).to(backend).train()
+    x = torch.randn(50, 12, device=backend)
+    close(stock(x, adj), dense_gen(stock, A, x), backend)
+    g_stock = grads_of(stock, stock(x, adj))
+    q = exact.QModule(torch.nn.ModuleList([stock])).model[0].to(backend).train()
+    assert type(q).__name__ == "QGENConv" and type(q.mlp).__name__ == "QMLP"
+    assert [type(m).__name__ for m in q.mlp] == ["QLinear", "QBatchNorm1d", "QReLU", "QDropout", "QLinear"]
+    assert isinstance(q.t, torch.nn.Parameter) == (learn and aggr == "softmax") and isinstance(q.p, torch.nn.Parameter) == learn
+    assert (q.msg_norm is not None) == msg_norm and q.eps == stock.eps
+    copy_params(q, stock)
+    config.compress_activation = False
+    close(q(x, adj), dense_gen(stock, A, x), backend)
+    g_q = grads_of(q, q(x, adj))
+    for k in g_stock:
+        close(g_q[k], g_stock[k], backend)
+    config.compress_activation = True
+    config.activation_compression_bits = [8]
+    q.zero_grad()
+    g_q8 = grads_of(q, q(x, adj))
+    for k in g_stock:
+        if g_stock[k].abs().max() > 1e-4:       # a bias in front of a batch norm has an exactly vanishing gradient
+            close(g_q8[k], g_stock[k], backend, loose=True)
+    with pytest.raises(NotImplementedError):
+        exact.QGENConv(4, 4, norm="layer")
