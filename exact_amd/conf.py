@@ -11,7 +11,7 @@ _REFERENCE_FIELDS = {
     "initial_bits": 8,
     "stochastic": True,                   # the kernels implement stochastic rounding only
     "use_gradient": False,
-    "simulate": False,                    # not provided here (raises when set)
+    "simulate": False,                    # the reference's tensor-op stand-in for the kernels (unpacked int32 codes)
     "enable_quantized_bn": True,          # QModule swaps BatchNorm1d only when set
     "kept_frac": 1.0,                     # < 1: random projection D -> int(kept_frac * D + 0.999)
     "single_precision": True,             # read at layer construction: attach QScheme objects

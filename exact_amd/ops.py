@@ -31,10 +31,19 @@ from .cpp_extension._checks import FLOAT_OR_HALF, check_device_tensor, ptr
 from .utils import empty_cache, swap_to_cpu
 
 
-def _unsupported_modes():
-    if config.simulate:
-        raise NotImplementedError("config.simulate (torch fake-quantisation, reference ops.py:21-34) is not "
-                                  "provided: this package only runs the packed kernels")
+def _simulated_quantize(data, bits, mn, mx):
+    """config.simulate (reference ops.py:18-31): the reference's debugging
+    stand-in for the kernels, plain tensor ops that keep the codes UNPACKED as
+    int32 [N, G] -- min / max widened by 1e-6, uniform(-0.5, 0.5) noise from
+    the torch generator, relu, round.  -> (codes, scale)."""
+    levels = 2 ** bits - 1
+    mn = mn - 1e-6
+    mx = mx + 1e-6
+    scale = levels / (mx - mn)
+    out = (data - mn.view(-1, 1)) * scale.view(-1, 1)
+    if config.stochastic:
+        out = out + torch.empty_like(out).uniform_(-0.5, 0.5)
+    return F.relu(out).round_().int(), scale
 
 
 def _rows_by_features(t):
@@ -55,7 +64,8 @@ def no_scheme_compute_quantization_bits(input):  # noqa: A002
 def quantize_and_pack(data, bits, mn, mx):
     """Two-step form with the row extrema given (reference ops.py:20-43):
     -> (packed int8 stream, fp32 scale)."""
-    _unsupported_modes()
+    if config.simulate:
+        return _simulated_quantize(data, bits, mn, mx)
     if type(bits) is not int:
         raise TypeError("bits must be an int")
     scale = (2 ** bits - 1) / (mx - mn)      # reciprocal() * int, as torch evaluates it
@@ -68,7 +78,9 @@ def quantize_and_pack(data, bits, mn, mx):
 def dequantize_and_unpack(data, shape, bits, scale, mn):
     """Reference ops.py:46-58; scale / min may be fp32 or the bf16 tensors that
     quantize_activation returned."""
-    _unsupported_modes()
+    if config.simulate:
+        scale, mn = scale.to(torch.float32), mn.to(torch.float32)
+        return data / scale.view(-1, 1) + mn.view(-1, 1)        # reference ops.py:47-48
     rows, feats = shape[0], math.prod(shape[1:])
     if data.device != scale.device:          # offloaded by config.swap (reference ops.py:50-51)
         data = data.to(scale.device, non_blocking=True)
@@ -82,11 +94,17 @@ def quantize_activation(input, scheme):  # noqa: A002
     bf16 casts are ONE kernel launch here."""
     if not config.compress_activation:
         return input, None, None, None
-    _unsupported_modes()
     if scheme:
         scheme.note_use()
     check_device_tensor(input, "input", None, FLOAT_OR_HALF)
     bits = config.activation_compression_bits[0]
+    if config.simulate:
+        flat = _rows_by_features(input)
+        lo, hi = ext_quantization.row_minmax(flat.float())
+        codes, scale = _simulated_quantize(flat, bits, lo.to(flat.dtype), hi.to(flat.dtype))
+        if input.dtype == torch.float32:
+            return codes, bits, scale.to(torch.bfloat16), lo.to(torch.bfloat16)
+        return codes, bits, scale, lo.to(flat.dtype)
     packed, scale_bf16, min_bf16 = ext_quantization.minmax_pack(_rows_by_features(input), bits)
     if config.swap:
         packed = swap_to_cpu(packed)
@@ -473,8 +491,7 @@ def relu_dropout(input, p, for_consumer=False):  # noqa: A002
     bits = None
     if (for_consumer and config.compress_activation and config.kept_frac == 1.0 and input.dim() == 2
             and input.dtype == torch.float32 and not torch.is_autocast_enabled()
-            and ext_quantization.fusable_width(input.shape[1])):
-        _unsupported_modes()
+            and not config.simulate and ext_quantization.fusable_width(input.shape[1])):
         bits = config.activation_compression_bits[0]
     out, packed, scale, mn = qrelu_dropout.apply(input, p, bits)
     if bits is not None:

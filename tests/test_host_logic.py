@@ -38,12 +38,9 @@ def test_install_as_exact_aliases_the_package():
     assert exact is exact_amd and q is extq and cfg is config
 
 
-def test_unsupported_modes_raise_instead_of_falling_back():
+def test_compression_off_passes_the_activation_through():
     x = torch.zeros(4, 4)
-    config.simulate = True
-    with pytest.raises(NotImplementedError, match="simulate"):
-        ops.quantize_activation(x, None)
-    config.simulate, config.compress_activation = False, False
+    config.compress_activation = False
     assert ops.quantize_activation(x, None) == (x, None, None, None)
     assert ops.dequantize_activation((x, None, None, None), x.shape) is x
 

@@ -371,3 +371,27 @@ def test_swap_keeps_the_packed_codes_on_the_host(backend):
         packed2, _ = ops.quantize_and_pack(x, 2, mn, mx)
         assert (packed2.device.type == "cpu") == (swap or backend.type == "cpu")
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+def test_simulate_mode(backend):
+    """config.simulate (reference ops.py:18-31, 47-48): unpacked int32 codes made
+    with tensor ops; within one level of the input, unbiased, usable by the layers."""
+    from exact_amd import ops
+    config.simulate = True
+    for bits in (2, 8):
+        config.activation_compression_bits = [bits]
+        x = torch.randn(300, 64, device=backend)
+        codes, qbits, scale, mn = ops.quantize_activation(x, None)
+        assert codes.dtype == torch.int32 and codes.shape == x.shape and qbits == bits
+        assert scale.dtype == torch.bfloat16 and int(codes.min()) >= 0 and int(codes.max()) <= 2 ** bits - 1
+        xh = ops.dequantize_activation((codes, qbits, scale, mn), x.shape)
+        step = (x.max(1).values - x.min(1).values) / (2 ** bits - 1)
+        assert ((xh - x).abs() <= 1.05 * step.unsqueeze(1) + 0.02 * x.abs().amax(1, keepdim=True)).all()
+    config.activation_compression_bits = [2]
+    draws = torch.stack([ops.dequantize_activation(ops.quantize_activation(x, None), x.shape) for _ in range(64)])
+    assert (draws.mean(0) - x).abs().mean() < 0.3 * (draws[0] - x).abs().mean()
+    packed, scale32 = ops.quantize_and_pack(x, 2, x.min(1).values, x.max(1).values)
+    assert packed.dtype == torch.int32 and scale32.dtype == torch.float32
+    lin = exact.QLinear(64, 8).to(backend).train()
+    lin(x.requires_grad_()).sum().backward()
+    assert torch.isfinite(lin.weight.grad).all() and torch.isfinite(x.grad).all()
