@@ -118,6 +118,7 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   constexpr int WPT = 8 / BITS;
   constexpr float B = static_cast<float>((1 << BITS) - 1);
   __shared__ uint2 stage[WPT > 1 ? OPT * kBlock : 1];
+  __shared__ f32x4 ybuf[ACT ? OPT * kBlock * 2 : 1];  // ACT: the activation output on its way to memory
 
   const int t = threadIdx.x;
   const int lpr = 1 << a.lpr_log2;
@@ -165,8 +166,32 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
           v[k][i] = r;
           m |= static_cast<uint32_t>(pos && keep) << i;
         }
-        store_oct<VEC, true>(a.y + row_off + d0, 8, v[k]);
+        // y leaves through LDS: an oct per lane would make every 16-byte store
+        // instruction skip every other 16 bytes, which halves the store rate
+        ybuf[(k * kBlock + t) * 2 + 0] = f32x4{v[k][0], v[k][1], v[k][2], v[k][3]};
+        ybuf[(k * kBlock + t) * 2 + 1] = f32x4{v[k][4], v[k][5], v[k][6], v[k][7]};
         a.mask_bytes[blk] = static_cast<uint8_t>(m);
+      }
+    }
+  }
+  if constexpr (ACT) {
+    // Lane l of a wavefront stores quad l, then quad 64 + l, of the wavefront's
+    // 64 octs of each k: whole runs of 32 * lpr contiguous bytes per row.
+    __syncthreads();
+    const int wave_first = t & ~(kWave - 1);
+#pragma unroll
+    for (int k = 0; k < OPT; ++k) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int q = s * kWave + (t & (kWave - 1));
+        const int src = wave_first + (q >> 1);  // the thread that produced this quad
+        const int half = q & 1;
+        const int64_t n_src = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (src >> a.lpr_log2);
+        const int j_src = (src & (lpr - 1)) + k * lpr;
+        if (n_src < a.N && j_src < a.opr) {
+          const f32x4 val = ybuf[(k * kBlock + src) * 2 + half];
+          nt_store4(a.y + n_src * a.G + 8 * j_src + 4 * half, val.x, val.y, val.z, val.w);
+        }
       }
     }
   }
