@@ -1,7 +1,13 @@
 """Drop-in quantised layers with the names, constructor arguments and
 forward signatures of exact/exact/layers.py in the reference (QLinear :268,
-QGCNConv :215, QSAGEConv :123, QBatchNorm1d :340, QReLU :284, QDropout :316,
-QDropout2 :328).  In eval mode every layer runs the stock op, as there."""
+QGCNConv :215, QSAGEConv :123, QGraphConv :181, QGCN2Conv :66, QGENConv :50,
+QMLP :32, QBatchNorm1d :340, QReLU :284, QLeakyReLU :295, QELU :304,
+QDropout :316, QDropout2 :328).  In eval mode a layer runs the stock op
+wherever the reference's does.
+
+Organisation (this library's own): the element-wise layers share one small
+base class that picks the training or the evaluation op; the convolutions get
+their QLinear / QMatmul parts from two helpers."""
 import torch
 import torch.nn.functional as F
 from torch.nn import Parameter
@@ -9,25 +15,66 @@ from torch.nn import Parameter
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCN2Conv, GCNConv, GENConv, GraphConv, SAGEConv, glorot
-from .ops import input2rp, qbatch_norm, qelu, qlinear, quantize_activation, relu_dropout, take_compressed
+from .ops import (input2rp, kept_columns, qbatch_norm, qelu, qlinear, quantize_activation, relu_dropout,
+                  take_compressed)
 from .qsheme import QScheme
 from .spmm import QMatmul, qmatmul
 
 
+def _scheme(name):
+    """Per-layer bookkeeping object of the reference (qsheme.py), attached only
+    when config.single_precision is set at construction time."""
+    return QScheme(name) if config.single_precision else None
+
+
+def _channel_pair(in_channels):
+    return (in_channels, in_channels) if isinstance(in_channels, int) else tuple(in_channels)
+
+
+# ---------------------------------------------------------------------------
+# linear
+# ---------------------------------------------------------------------------
 class QLinear(torch.nn.Linear):
     def __init__(self, input_features, output_features, bias=True, rp=True):
         super().__init__(input_features, output_features, bias)
-        self.scheme = QScheme("linear") if config.single_precision else None
+        self.scheme = _scheme("linear")
         self.rp = rp
 
     def forward(self, input, quantized=None, randmat=None):  # noqa: A002
-        if self.training:
-            if quantized is None:
-                quantized = take_compressed(input, project=self.rp)
-            return qlinear.apply(input, self.weight, self.bias, quantized, randmat, self.scheme, self.rp)
-        return super().forward(input)
+        if not self.training:
+            return super().forward(input)
+        if quantized is None:
+            quantized = take_compressed(input, project=self.rp)   # a copy a fused producer made, if any
+        return qlinear.apply(input, self.weight, self.bias, quantized, randmat, self.scheme, self.rp)
 
 
+def qaddmm(input, mat1, mat2, beta=1.0, alpha=1):  # noqa: A002
+    """layers.py:27-28.  As there, the product is qlinear(mat1, mat2) = mat1 @
+    mat2^T (not torch.addmm's mat1 @ mat2): QGCN2Conv multiplies by the
+    transposed weight in the reference, and so does this."""
+    return beta * input + alpha * qlinear.apply(mat1, mat2, None)
+
+
+class QMLP(torch.nn.Sequential):
+    """layers.py:32-47: QLinear (-> QBatchNorm1d) -> QReLU -> QDropout blocks."""
+
+    def __init__(self, channels, norm, bias=True, dropout=0.0):
+        if norm and norm != "batch":
+            raise NotImplementedError(f'Normalization layer "{norm}" not supported.')
+        widths = list(zip(channels[:-1], channels[1:]))
+        blocks = []
+        for index, (fan_in, fan_out) in enumerate(widths):
+            blocks.append(QLinear(fan_in, fan_out, bias))
+            if index + 1 < len(widths):                 # every layer but the last
+                if norm:
+                    blocks.append(QBatchNorm1d(fan_out, affine=True))
+                blocks += [QReLU(), QDropout(dropout)]
+        super().__init__(*blocks)
+
+
+# ---------------------------------------------------------------------------
+# convolutions
+# ---------------------------------------------------------------------------
 class QGCNConv(GCNConv):
     """layers.py:215-265: the weight is stored [out, in] and the linear map is
     a qlinear; propagation is a quantised SpMM."""
@@ -36,7 +83,7 @@ class QGCNConv(GCNConv):
         super().__init__(*args, **kwargs)
         self.weight = Parameter(torch.Tensor(self.out_channels, self.in_channels))
         self.msg_and_aggr_func = QMatmul(self.aggr)
-        self.lin_scheme = QScheme("linear") if config.single_precision else None
+        self.lin_scheme = _scheme("linear")
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -45,22 +92,31 @@ class QGCNConv(GCNConv):
             self.bias.data.zero_()
         self._cached_adj_t = None
 
+    def _transform(self, x):
+        if not self.training:
+            return F.linear(x, self.weight, None)
+        # layers.py:252 passes lin_scheme in the `randmat` slot; with
+        # kept_frac == 1 that slot is unused, so the numbers are those of a
+        # qlinear without a scheme.  Here the scheme is passed as scheme.
+        return qlinear.apply(x, self.weight, None, take_compressed(x), None, self.lin_scheme)
+
     def forward(self, x, edge_index, edge_weight=None):
         adj_t = self._normalized(edge_index)
-        if self.training:
-            # layers.py:252 passes lin_scheme in the `randmat` slot; with
-            # kept_frac == 1 that slot is unused, so the numbers are those of
-            # a qlinear without a scheme.  Here the scheme is passed as scheme.
-            x = qlinear.apply(x, self.weight, None, take_compressed(x), None, self.lin_scheme)
-        else:
-            x = F.linear(x, self.weight, None)
-        out = self.message_and_aggregate(adj_t, x)
-        if self.bias is not None:
-            out = out + self.bias
-        return out
+        out = self.message_and_aggregate(adj_t, self._transform(x))
+        return out if self.bias is None else out + self.bias
 
     def message_and_aggregate(self, adj_t, x):
         return self.msg_and_aggr_func(adj_t, x)
+
+
+def _quantise_two_linears(conv, root_optional):
+    """lin_l / lin_r of a SAGE- or GraphConv-style layer as QLinear, plus the
+    quantised aggregation (layers.py:124-139, 182-191)."""
+    fan_l, fan_r = _channel_pair(conv.in_channels)
+    conv.lin_l = QLinear(fan_l, conv.out_channels, bias=conv.lin_l.bias is not None, rp=True)
+    if not root_optional or conv.root_weight:
+        conv.lin_r = QLinear(fan_r, conv.out_channels, bias=False, rp=True)
+    conv.msg_and_aggr_func = QMatmul(conv.aggr)
 
 
 class QSAGEConv(SAGEConv):
@@ -69,40 +125,28 @@ class QSAGEConv(SAGEConv):
 
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
-        in_channels = self.in_channels
-        if isinstance(in_channels, int):
-            in_channels = (in_channels, in_channels)
-        bias = self.lin_l.bias is not None
-        self.lin_l = QLinear(in_channels[0], self.out_channels, bias=bias, rp=True)
-        if self.root_weight:
-            self.lin_r = QLinear(in_channels[1], self.out_channels, bias=False, rp=True)
-        self.msg_and_aggr_func = QMatmul(self.aggr)
-        self.scheme = QScheme("sage") if config.single_precision else None
+        _quantise_two_linears(self, root_optional=True)
+        self.scheme = _scheme("sage")
         self.reset_parameters()
 
+    def _shared_copy(self, x):
+        """-> (quantized, randmat) of x for both consumers (layers.py:153-159)."""
+        handed_over = take_compressed(x)
+        if handed_over is not None:
+            return handed_over, None
+        if config.kept_frac < 1.0:
+            reduced, randmat = input2rp(x, kept_columns(x.shape[1]))
+            return quantize_activation(reduced, self.scheme), randmat
+        return quantize_activation(x, self.scheme), None
+
     def forward(self, x, edge_index, size=None):
-        if isinstance(x, torch.Tensor):
-            x = (x, x)
-            l_eq_r = True
-        else:
-            l_eq_r = False
-        if l_eq_r and self.training:
-            if config.kept_frac < 1.0:
-                kept_acts = int(config.kept_frac * x[0].shape[1] + 0.999)
-                dim_reduced_input, randmat = input2rp(x[0], kept_acts)
-            else:
-                dim_reduced_input, randmat = x[0], None
-            quantized = take_compressed(x[0]) or quantize_activation(dim_reduced_input, self.scheme)
-        else:
-            quantized, randmat = None, None
-        out = self.message_and_aggregate(edge_index, x, quantized=quantized, randmat=randmat)
-        out = self.lin_l(out)
-        x_r = x[1]
+        same_both_sides = isinstance(x, torch.Tensor)
+        x_l, x_r = (x, x) if same_both_sides else x
+        quantized, randmat = self._shared_copy(x_l) if (same_both_sides and self.training) else (None, None)
+        out = self.lin_l(self.message_and_aggregate(edge_index, (x_l, x_r), quantized=quantized, randmat=randmat))
         if self.root_weight and x_r is not None:
             out = out + self.lin_r(x_r, quantized, randmat)
-        if self.normalize:
-            out = F.normalize(out, p=2.0, dim=-1)
-        return out
+        return F.normalize(out, p=2.0, dim=-1) if self.normalize else out
 
     def message_and_aggregate(self, adj_t, x, quantized=None, randmat=None):
         return self.msg_and_aggr_func(adj_t, x[0], quantized=quantized, randmat=randmat)
@@ -114,24 +158,11 @@ class QGraphConv(GraphConv):
 
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
-        in_channels = self.in_channels
-        if isinstance(in_channels, int):
-            in_channels = (in_channels, in_channels)
-        bias = self.lin_l.bias is not None
-        self.lin_l = QLinear(in_channels[0], self.out_channels, bias=bias, rp=True)
-        self.lin_r = QLinear(in_channels[1], self.out_channels, bias=False, rp=True)
-        self.msg_and_aggr_func = QMatmul(self.aggr)
+        _quantise_two_linears(self, root_optional=False)
         self.reset_parameters()
 
     def message_and_aggregate(self, adj_t, x):
         return self.msg_and_aggr_func(adj_t, x[0])
-
-
-def qaddmm(input, mat1, mat2, beta=1.0, alpha=1):  # noqa: A002
-    """layers.py:27-28.  As there, the product is qlinear(mat1, mat2) = mat1 @
-    mat2^T (not torch.addmm's mat1 @ mat2): QGCN2Conv multiplies by the
-    transposed weight in the reference, and so does this."""
-    return beta * input + alpha * qlinear.apply(mat1, mat2, None)
 
 
 class QGCN2Conv(GCN2Conv):
@@ -142,23 +173,6 @@ class QGCN2Conv(GCN2Conv):
 
     def _addmm(self, inp, mat, weight):
         return qaddmm(inp, mat, weight, beta=1.0 - self.beta, alpha=self.beta)
-
-
-class QMLP(torch.nn.Sequential):
-    """layers.py:32-47: QLinear (-> QBatchNorm1d) -> QReLU -> QDropout blocks."""
-
-    def __init__(self, channels, norm, bias=True, dropout=0.0):
-        blocks = []
-        for i in range(1, len(channels)):
-            blocks.append(QLinear(channels[i - 1], channels[i], bias))
-            if i < len(channels) - 1:
-                if norm == "batch":
-                    blocks.append(QBatchNorm1d(channels[i], affine=True))
-                elif norm:
-                    raise NotImplementedError(f'Normalization layer "{norm}" not supported.')
-                blocks.append(QReLU())
-                blocks.append(QDropout(dropout))
-        super().__init__(*blocks)
 
 
 class QGENConv(GENConv):
@@ -172,63 +186,80 @@ class QGENConv(GENConv):
         return ext_quantization.act_quantized_relu(msg) + self.eps
 
 
-class QReLU(torch.nn.Module):
+# ---------------------------------------------------------------------------
+# element-wise layers: a compressed op in training, the stock op in evaluation
+# ---------------------------------------------------------------------------
+class _TrainEval(torch.nn.Module):
+    always_compressed = False        # QLeakyReLU keeps its mask in eval mode as well (layers.py:300-301)
+
+    def _train(self, t):
+        raise NotImplementedError
+
+    def _eval(self, t):
+        raise NotImplementedError
+
+    def forward(self, input):  # noqa: A002
+        return self._train(input) if (self.training or self.always_compressed) else self._eval(input)
+
+
+class QReLU(_TrainEval):
     def __init__(self, inplace=False):
         super().__init__()
 
-    def forward(self, input):  # noqa: A002
-        if self.training:
-            return ext_quantization.act_quantized_relu(input)
-        return F.relu(input)
+    def _train(self, t):
+        return ext_quantization.act_quantized_relu(t)
+
+    def _eval(self, t):
+        return F.relu(t)
 
 
-class QLeakyReLU(torch.nn.Module):
-    """layers.py:295-301 of the reference (compressed in train and eval alike)."""
+class QLeakyReLU(_TrainEval):
+    always_compressed = True
 
     def __init__(self, negative_slope, inplace=False):
         super().__init__()
         self.negative_slope = negative_slope
 
-    def forward(self, input):  # noqa: A002
-        return ext_quantization.act_quantized_leaky_relu(input, self.negative_slope)
+    def _train(self, t):
+        return ext_quantization.act_quantized_leaky_relu(t, self.negative_slope)
 
 
-class QELU(torch.nn.Module):
-    """layers.py:304-313 of the reference."""
-
+class QELU(_TrainEval):
     def __init__(self, alpha, inplace=False):
         super().__init__()
         self.alpha = alpha
 
-    def forward(self, input):  # noqa: A002
-        if self.training:
-            return qelu.apply(input, self.alpha)
-        return F.elu(input, self.alpha)
+    def _train(self, t):
+        return qelu.apply(t, self.alpha)
+
+    def _eval(self, t):
+        return F.elu(t, self.alpha)
 
 
-class QDropout(torch.nn.Module):
+class QDropout(_TrainEval):
     def __init__(self, p):
         super().__init__()
         self.p = p
 
-    def forward(self, input):  # noqa: A002
-        if self.training:
-            return ext_quantization.act_quantized_dropout(input, self.p, self.training)
-        return F.dropout(input, self.p, self.training)
+    def _train(self, t):
+        return ext_quantization.act_quantized_dropout(t, self.p, True)
+
+    def _eval(self, t):
+        return t                      # F.dropout(t, p, training=False)
 
 
-class QDropout2(torch.nn.Module):
-    def __init__(self, p):
-        super().__init__()
-        self.p = p
+class QDropout2(QDropout):
+    """layers.py:328-337: dropout whose survivors keep their magnitude (the
+    1 / (1 - p) of dropout is undone); evaluation scales by (1 - p)."""
 
-    def forward(self, input):  # noqa: A002
-        if self.training:
-            return ext_quantization.act_quantized_dropout(input, self.p, self.training) * (1 - self.p)
-        return F.dropout(input, self.p, self.training) * (1 - self.p)
+    def _train(self, t):
+        return super()._train(t) * (1 - self.p)
+
+    def _eval(self, t):
+        return t * (1 - self.p)
 
 
-class QReLUDropout(torch.nn.Module):
+class QReLUDropout(_TrainEval):
     """QReLU followed by QDropout (layers.py:284-325) as one pass that keeps one
     joint mask; with `for_consumer`, the compressed copy the following
     QLinear / QGCNConv / QSAGEConv would make of the result is produced in the
@@ -239,10 +270,11 @@ class QReLUDropout(torch.nn.Module):
         self.p = p
         self.for_consumer = for_consumer
 
-    def forward(self, input):  # noqa: A002
-        if self.training:
-            return relu_dropout(input, self.p, self.for_consumer)
-        return F.relu(input)
+    def _train(self, t):
+        return relu_dropout(t, self.p, self.for_consumer)
+
+    def _eval(self, t):
+        return F.relu(t)
 
     def extra_repr(self):
         return f"p={self.p}, for_consumer={self.for_consumer}"
@@ -251,19 +283,22 @@ class QReLUDropout(torch.nn.Module):
 class QBatchNorm1d(torch.nn.BatchNorm1d):
     def __init__(self, num_features, eps=1e-05, momentum=0.1, affine=True, track_running_stats=True):
         super().__init__(num_features, eps, momentum, affine, track_running_stats)
-        self.scheme = QScheme("batchnorm") if config.single_precision else None
+        self.scheme = _scheme("batchnorm")
+
+    def _averaging_factor(self):
+        """Weight of this batch in the running statistics; counts the batch
+        (torch.nn.BatchNorm1d's bookkeeping, layers.py:352-369)."""
+        if not (self.track_running_stats and self.num_batches_tracked is not None):
+            return 0.0 if self.momentum is None else self.momentum
+        self.num_batches_tracked = self.num_batches_tracked + 1
+        if self.momentum is None:                       # cumulative moving average
+            return 1.0 / float(self.num_batches_tracked)
+        return self.momentum
 
     def forward(self, input):  # noqa: A002
         if not self.training:
             return super().forward(input)
         self._check_input_dim(input)
-        exponential_average_factor = 0.0 if self.momentum is None else self.momentum
-        if self.track_running_stats and self.num_batches_tracked is not None:
-            self.num_batches_tracked = self.num_batches_tracked + 1
-            if self.momentum is None:
-                exponential_average_factor = 1.0 / float(self.num_batches_tracked)
-        return qbatch_norm.apply(
-            input,
-            self.running_mean if self.track_running_stats else None,
-            self.running_var if self.track_running_stats else None,
-            self.weight, self.bias, True, exponential_average_factor, self.eps, self.scheme)
+        factor = self._averaging_factor()
+        running = (self.running_mean, self.running_var) if self.track_running_stats else (None, None)
+        return qbatch_norm.apply(input, *running, self.weight, self.bias, True, factor, self.eps, self.scheme)
