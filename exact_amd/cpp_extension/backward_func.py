@@ -1,8 +1,11 @@
 """Stand-in for the reference's `exact.cpp_extension.backward_func` module
 (backward_func.cc:83-107).  The reference only re-exports ATen routines plus
-the two-GEMM linear backward; the same ATen routines are reachable from
-Python, so no native code is needed here."""
+the two-GEMM linear backward, which are reachable from Python as they are;
+its one kernel of its own, the ELU derivative, is a kernel of the library."""
 import torch
+
+from .. import _lib
+from . import _checks
 
 
 def linear_backward(grad_output, input, weight, bias):  # noqa: A002
@@ -25,4 +28,14 @@ def native_batch_norm_backward(grad_out, input, weight, running_mean, running_va
 
 def _elu_backward_cuda(grad_output, data, alpha):
     """backward_func_cuda_kernel.cu:6-36: x >= 0 ? grad : alpha * grad * exp(x)."""
-    return torch.where(data >= 0, grad_output, alpha * grad_output * torch.exp(data))
+    grad_output, data = grad_output.contiguous(), data.contiguous()
+    _checks.check_device_tensor(grad_output, "grad_output", None, _checks.FLOAT_OR_HALF)
+    _checks.check_device_tensor(data, "data", None, (grad_output.dtype,))
+    if data.numel() != grad_output.numel():
+        raise RuntimeError("grad_output and data must have the same number of elements")
+    grad_input = torch.empty_like(grad_output)
+    fn = getattr(_lib.lib(), "exact_elu_bwd_" + _checks.suffix(grad_output))
+    rc = fn(_checks.ptr(grad_output), _checks.ptr(data), float(alpha), grad_output.numel(), _checks.ptr(grad_input),
+            _checks.stream_ptr(grad_output))
+    _lib.check(rc, "_elu_backward_cuda")
+    return grad_input

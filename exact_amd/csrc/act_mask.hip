@@ -257,6 +257,29 @@ __global__ __launch_bounds__(kBlock) void dropout_bwd_kernel(const T* __restrict
   }
 }
 
+// ELU backward on the (decompressed) input: dx = x >= 0 ? dy : alpha * dy * exp(x)
+// (backward_func_cuda_kernel.cu:6-20; alpha * dy first, then the exponential).
+template <bool VEC4, typename T>
+__global__ __launch_bounds__(kBlock) void elu_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                                         float alpha, int64_t n, T* __restrict__ dx) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t quad = static_cast<int64_t>(blockIdx.x) * kTileQuads + h * kBlock + threadIdx.x;
+    const int nv = valid_in_quad(quad, n);
+    if (nv == 0) continue;
+    float g[4], v[4];
+    load4<VEC4>(dy + quad * 4, nv, g);
+    load4<VEC4>(x + quad * 4, nv, v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float scaled = alpha * g[i];
+      scaled = scaled * expf(v[i]);
+      g[i] = v[i] >= 0.f ? g[i] : scaled;
+    }
+    store4<VEC4>(dx + quad * 4, nv, g);
+  }
+}
+
 // a quad of T is one aligned vector access
 template <typename T>
 static bool quad_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & (4 * sizeof(T) - 1)) == 0; }
@@ -361,6 +384,19 @@ static int dropout_backward(const T* dy, const uint32_t* mask, float p, int64_t 
   return launch_status();
 }
 
+template <typename T>
+static int elu_backward(const T* dy, const T* x, float alpha, int64_t n, T* dx, void* stream) {
+  if (int rc = check_n(n)) return rc;
+  if (n == 0) return EXACT_OK;
+  if (!dy || !x || !dx) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (quad_aligned<T>(dy) && quad_aligned<T>(x) && quad_aligned<T>(dx))
+    hipLaunchKernelGGL((elu_bwd_kernel<true, T>), tile_grid(n), dim3(kBlock), 0, s, dy, x, alpha, n, dx);
+  else
+    hipLaunchKernelGGL((elu_bwd_kernel<false, T>), tile_grid(n), dim3(kBlock), 0, s, dy, x, alpha, n, dx);
+  return launch_status();
+}
+
 }  // namespace exact
 
 using namespace exact;
@@ -394,6 +430,13 @@ int exact_relu_dropout_fwd_f32(const float* x, const float* noise, uint64_t seed
 int exact_dropout_bwd_f32(const float* dy, const uint32_t* mask, float p, int64_t n, float* dx,
                           void* stream) {
   return dropout_backward<float>(dy, mask, p, n, dx, stream);
+}
+
+int exact_elu_bwd_f32(const float* dy, const float* x, float alpha, int64_t n, float* dx, void* stream) {
+  return elu_backward<float>(dy, x, alpha, n, dx, stream);
+}
+int exact_elu_bwd_f16(const uint16_t* dy, const uint16_t* x, float alpha, int64_t n, uint16_t* dx, void* stream) {
+  return elu_backward<half_t>(hp(dy), hp(x), alpha, n, hp(dx), stream);
 }
 
 // fp16 activations: the same kernels instantiated for 16-bit elements

@@ -150,6 +150,14 @@ int exact_leaky_relu_fwd_f32(const float *x, int64_t n, float slope, float *y,
 int exact_leaky_relu_bwd_f32(const float *dy, const uint32_t *mask, int64_t n,
                              float slope, float *dx, void *stream);
 
+/* ELU backward on the decompressed input: dx = x >= 0 ? dy : alpha * dy * exp(x).
+ * Replaces _elu_backward_cuda (backward_func_cuda_kernel.cu:6-36) as called by
+ * qelu.backward (ops.py:195-203).  exact_elu_bwd_f16: the same on fp16 tensors. */
+int exact_elu_bwd_f32(const float *dy, const float *x, float alpha, int64_t n,
+                      float *dx, void *stream);
+int exact_elu_bwd_f16(const uint16_t *dy, const uint16_t *x, float alpha, int64_t n,
+                      uint16_t *dx, void *stream);
+
 /* Fused epilogues (no single counterpart in the reference: each replaces a
  * chain of its calls with one pass over the data, bit-identical to the chain).
  *

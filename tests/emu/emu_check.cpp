@@ -255,6 +255,14 @@ static void check_leaky(int64_t n, std::mt19937& rng) {
   }
   for (int64_t i = n; i < words * 32; ++i) bad += (m[i / 32] >> (i % 32)) & 1u;  // tail bits are written as 0
   CHECK(bad == 0, "leaky relu differs n=%ld: %ld", (long)n, (long)bad);
+  // ELU derivative on the same data
+  CHECK(exact_elu_bwd_f32(g.p, x.p, 1.3f, n, dx.p, nullptr) == 0, "elu bwd rc");
+  bad = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    const float want = x[i] >= 0.f ? g[i] : (1.3f * g[i]) * std::exp(x[i]);
+    bad += std::fabs(dx[i] - want) > 4e-7f * std::fabs(want);
+  }
+  CHECK(bad == 0, "elu backward differs n=%ld: %ld", (long)n, (long)bad);
 }
 
 // ReLU -> dropout (-> statistics + pack) in one pass against the chain of the

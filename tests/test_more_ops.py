@@ -395,3 +395,23 @@ def test_simulate_mode(backend):
     lin = exact.QLinear(64, 8).to(backend).train()
     lin(x.requires_grad_()).sum().backward()
     assert torch.isfinite(lin.weight.grad).all() and torch.isfinite(x.grad).all()
+
+
+def test_elu_backward_kernel(backend):
+    """_elu_backward_cuda (backward_func_cuda_kernel.cu:6-36) as a kernel of the
+    library, fp32 and fp16, against the formula (exp within 2 ulp)."""
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator().manual_seed(3)
+    for n in (1, 7, 1000, 4099):
+        x = (torch.randn(n, generator=g) * 2).to(backend)
+        x[::5] = 0.0
+        dy = torch.randn(n, generator=g).to(backend)
+        got = bf._elu_backward_cuda(dy, x, 1.3)
+        want = torch.where(x >= 0, dy, (1.3 * dy) * torch.exp(x))
+        assert torch.equal(got[x >= 0], dy[x >= 0])
+        assert torch.allclose(got, want, rtol=3e-7, atol=0)
+        got_h = bf._elu_backward_cuda(dy.half(), x.half(), 1.3)
+        want_h = torch.where(x.half() >= 0, dy.half(), ((1.3 * dy.half().float()) * torch.exp(x.half().float())).half())
+        assert got_h.dtype == torch.float16 and (got_h.float() - want_h.float()).abs().max() <= 2e-3 * want_h.float().abs().max()
+    with pytest.raises(RuntimeError):
+        bf._elu_backward_cuda(dy, x[:-1], 1.0)
