@@ -120,10 +120,21 @@ def main(argv=None):
     seed = 0x5EED
     calls = [0]
 
+    # Work split of the pack kernel: the library times its alternatives (1, 2 or 4
+    # column groups per lane, same result) once per (width, bits) and keeps the fastest.
+    from exact_amd.cpp_extension import quantization as extq
+    geometry = {"octs_per_lane": {}, "candidates_us": {}}
+    for b in BITS:
+        if x.is_cuda:
+            tried = extq.tune_pack_geometry(x, b)
+            geometry["candidates_us"][str(b)] = {str(c): t * 1e6 for c, t in tried.items()}
+        geometry["octs_per_lane"][str(b)] = extq._PACK_GEOMETRY.get((G, b), 0)
+    log(f"pack work split (octs per lane) by bits: {geometry['octs_per_lane']}  timings (us): {geometry['candidates_us']}")
+
     def pack(b):
         calls[0] += 1
-        rc = L.exact_minmax_pack_f32(x.data_ptr(), None, seed, calls[0], N, G, b, packed[b].data_ptr(), None, None,
-                                     sbf.data_ptr(), mbf.data_ptr(), sp)
+        rc = L.exact_minmax_pack_geom_f32(x.data_ptr(), None, seed, calls[0], N, G, b, packed[b].data_ptr(), None,
+                                          None, sbf.data_ptr(), mbf.data_ptr(), geometry["octs_per_lane"][str(b)], sp)
         assert rc == 0, rc
 
     def unpack(b):
@@ -200,7 +211,7 @@ def main(argv=None):
                    "rows": N, "cols": G, "bits": list(BITS), "algo_bytes_per_step": step_bytes},
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBS,
         "epochs_per_s": {k: v.get("epochs_per_s") for k, v in extras.items() if isinstance(v, dict) and k.startswith("cfg")},
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "extras": extras,
+        "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "pack_geometry": geometry, "extras": extras,
     }
     print(json.dumps(result), flush=True)
     return result

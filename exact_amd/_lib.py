@@ -27,6 +27,7 @@ SIGNATURES = {
     "exact_row_minmax_f32": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr]),
     "exact_pack_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
     "exact_minmax_pack_f32": (_c_int, [_c_ptr, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
+    "exact_minmax_pack_geom_f32": (_c_int, [_c_ptr, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "exact_unpack_f32": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_unpack_bf16param_f32": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_relu_fwd_f32": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr]),

@@ -47,6 +47,10 @@ _EXTRA_FIELDS = {
     # model offers the pair as one module (QReLUDropout).  Results are
     # bit-identical to the separate layers; False runs them separately.
     "fuse_epilogue": True,
+    # Time the alternative work splits of the pack kernel (1, 2 or 4 column
+    # groups per lane) the first time a large activation of a new (width, bits)
+    # is compressed on a GPU, and keep the fastest.  Results do not depend on it.
+    "autotune_pack": True,
 }
 
 

@@ -77,6 +77,57 @@ def unpack_single_precision(data, bits, scale, min, N, group_size):  # noqa: A00
     return out
 
 
+# ---- work split of the fused pack kernel ---------------------------------------
+# (G, bits) -> octs per lane found fastest by tune_pack_geometry; 0 or absent = the library's default
+_PACK_GEOMETRY = {}
+_TUNE_MIN_ELEMENTS = 1 << 20
+
+
+def pack_geometry_candidates(G):
+    """Octs (8-column groups) per lane the kernel accepts for rows of G columns."""
+    octs = (G + 7) // 8
+    return [c for c in (1, 2, 4) if (octs + c - 1) // c <= 32 and (c == 1 or octs >= c)]
+
+
+def tune_pack_geometry(data, bits, reps=5):
+    """Time exact_minmax_pack_geom_f32 on `data` (read only; outputs go to
+    scratch buffers, no random numbers are consumed) with every candidate split,
+    remember the fastest for (G, bits) and return {candidate: seconds}."""
+    N, G = data.shape
+    dev = data.device
+    packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=dev)
+    scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    stream = _checks.stream_ptr(data)
+    fn = _lib.lib().exact_minmax_pack_geom_f32
+    timings = {}
+    for cand in pack_geometry_candidates(G):
+        def launch():
+            rc = fn(ptr(data), None, 0x7E57, 4, N, G, bits, ptr(packed), None, None, ptr(scale_bf), ptr(min_bf), cand, stream)
+            _lib.check(rc, "tune_pack_geometry")
+        launch()                                            # warm-up (first touch, code load)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            launch()
+        stop.record()
+        stop.synchronize()
+        timings[cand] = start.elapsed_time(stop) * 1e-3 / reps
+    _PACK_GEOMETRY[(G, bits)] = min(timings, key=timings.get)
+    return timings
+
+
+def _pack_geometry(data, bits):
+    """The split to ask for: the remembered one, after tuning when that is due."""
+    key = (data.shape[1], bits)
+    if key not in _PACK_GEOMETRY:
+        if not (config.autotune_pack and data.is_cuda and data.numel() >= _TUNE_MIN_ELEMENTS
+                and len(pack_geometry_candidates(key[0])) > 1) or torch.cuda.is_current_stream_capturing():
+            return 0
+        tune_pack_geometry(data, bits)
+    return _PACK_GEOMETRY[key]
+
+
 # ---- fused forms (no counterpart module function in the reference) ----------
 def minmax_pack(data, bits, want_fp32=False):
     """One pass over data[N, G]: per-row min and scale (ops.py:39, 61-66),
@@ -106,9 +157,9 @@ def minmax_pack(data, bits, want_fp32=False):
     scale32 = torch.empty(N, dtype=torch.float32, device=dev) if need32 else None
     min32 = torch.empty(N, dtype=torch.float32, device=dev) if need32 else None
     noise, seed, offset = _noise_for(data.shape, dev)
-    rc = _lib.lib().exact_minmax_pack_f32(ptr(data), ptr(noise), seed, offset, N, G, bits, ptr(packed),
-                                          ptr(scale32), ptr(min32), ptr(scale_bf), ptr(min_bf),
-                                          _checks.stream_ptr(data))
+    rc = _lib.lib().exact_minmax_pack_geom_f32(ptr(data), ptr(noise), seed, offset, N, G, bits, ptr(packed),
+                                               ptr(scale32), ptr(min32), ptr(scale_bf), ptr(min_bf),
+                                               _pack_geometry(data, bits), _checks.stream_ptr(data))
     _lib.check(rc, "minmax_pack")
     if want_fp32:
         return packed, scale_bf, min_bf, scale32, min32

@@ -360,7 +360,9 @@ struct Geometry {
 
 // Octs per thread and lanes per row for rows of G columns.  `max_opt` octs fit
 // in registers; longer rows are tiled over grid.y (two-step form only).
-static Geometry plan_rows(int64_t G, int max_opt) {
+// `opt_hint` (1, 2 or 4; 0 = none) overrides the default choice when the row
+// still fits 32 lanes with it: the caller may have timed the alternatives.
+static Geometry plan_rows(int64_t G, int max_opt, int opt_hint = 0) {
   Geometry g;
   g.opr = static_cast<int>((G + 7) / 8);
   // Aim for 16 lanes per row: the per-lane fixed work (row statistics butterfly,
@@ -370,6 +372,9 @@ static Geometry plan_rows(int64_t G, int max_opt) {
   if (opt > max_opt) opt = max_opt;
   if (opt == 3) opt = 4;
   if (opt < 1) opt = 1;
+  if ((opt_hint == 1 || opt_hint == 2 || opt_hint == 4) && opt_hint <= max_opt &&
+      (g.opr + opt_hint - 1) / opt_hint <= 32)
+    opt = opt_hint;
   const int lanes_needed = (g.opr + opt - 1) / opt;
   int l2 = 0;
   while ((1 << l2) < lanes_needed && l2 < 5) ++l2;
@@ -423,7 +428,7 @@ static int check_quant_shape(int64_t N, int64_t G, int bits) {
 static int pack_common(const float* x, const float* mn, const float* scale, const float* noise,
                        uint64_t seed, uint64_t offset, int64_t N, int64_t G, int bits,
                        uint8_t* packed, float* scale_f32, float* min_f32, uint16_t* scale_bf16,
-                       uint16_t* min_bf16, bool fused, hipStream_t s) {
+                       uint16_t* min_bf16, bool fused, hipStream_t s, int opt_hint = 0) {
   if (int rc = check_quant_shape(N, G, bits)) return rc;
   if (!packed) return EXACT_E_NULL;
   const int64_t pad_index = exact_packed_nbytes(N, G, bits) - 1;
@@ -453,7 +458,7 @@ static int pack_common(const float* x, const float* mn, const float* scale, cons
     do_fused = false;
   }
 
-  const Geometry g = plan_rows(G, do_fused ? 4 : 1);
+  const Geometry g = plan_rows(G, do_fused ? 4 : 1, opt_hint);
   PackArgs a{};
   a.x = x;
   a.noise = noise;
@@ -584,6 +589,15 @@ int exact_minmax_pack_f32(const float* x, const float* noise, uint64_t seed, uin
                           float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, void* stream) {
   return pack_common(x, nullptr, nullptr, noise, seed, offset, N, G, bits, packed, scale_f32, min_f32,
                      scale_bf16, min_bf16, true, static_cast<hipStream_t>(stream));
+}
+
+int exact_minmax_pack_geom_f32(const float* x, const float* noise, uint64_t seed, uint64_t offset,
+                               int64_t N, int64_t G, int bits, uint8_t* packed, float* scale_f32,
+                               float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, int octs_per_lane,
+                               void* stream) {
+  if (octs_per_lane != 0 && octs_per_lane != 1 && octs_per_lane != 2 && octs_per_lane != 4) return EXACT_E_ARG;
+  return pack_common(x, nullptr, nullptr, noise, seed, offset, N, G, bits, packed, scale_f32, min_f32,
+                     scale_bf16, min_bf16, true, static_cast<hipStream_t>(stream), octs_per_lane);
 }
 
 int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act_noise, uint64_t act_seed,

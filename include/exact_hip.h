@@ -77,6 +77,17 @@ int exact_minmax_pack_f32(const float *x, const float *noise, uint64_t seed,
                           uint8_t *packed, float *scale_f32, float *min_f32,
                           uint16_t *scale_bf16, uint16_t *min_bf16, void *stream);
 
+/* The same with the work split chosen by the caller: octs_per_lane = 1, 2 or 4
+ * consecutive 8-column groups per lane (0 = the library's default; a value the
+ * row length does not allow is ignored).  The result does not depend on it;
+ * the host side times the alternatives once per (G, bits) and keeps the
+ * fastest. */
+int exact_minmax_pack_geom_f32(const float *x, const float *noise, uint64_t seed,
+                               uint64_t offset, int64_t N, int64_t G, int bits,
+                               uint8_t *packed, float *scale_f32, float *min_f32,
+                               uint16_t *scale_bf16, uint16_t *min_bf16,
+                               int octs_per_lane, void *stream);
+
 /* a5. Unpack + dequantise: out[n, d] = float(field) / scale[n] + mn[n].
  * Replaces unpack_single_precision(data, bits, scale, min, N, group_size)
  * (quantization.cc:50-62 -> quantization_cuda_kernel.cu:158-229). */

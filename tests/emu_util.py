@@ -313,3 +313,20 @@ def mask_bwd_f16(kind, dy, mask, arg=None):
         rc = emu().exact_dropout_bwd_f16(p(dy), p(mask), arg, dy.size, p(dx), None)
     assert rc == 0, rc
     return dx
+
+
+def minmax_pack_geom(x, bits, octs_per_lane, noise=None, seed=0, offset=0, guard=64, expect_rc=0):
+    """exact_minmax_pack_geom_f32 -> (packed, scale bf16 bits, min bf16 bits)."""
+    x = f32(x)
+    N, G = x.shape
+    nb = int(emu().exact_packed_nbytes(N, G, bits))
+    packed = np.full(nb + guard, 0xA5, np.uint8)
+    sbf, mbf = np.zeros(N, np.uint16), np.zeros(N, np.uint16)
+    noise = None if noise is None else f32(noise)
+    rc = emu().exact_minmax_pack_geom_f32(p(x), p(noise), seed, offset, N, G, bits, p(packed), None, None, p(sbf),
+                                          p(mbf), octs_per_lane, None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (packed[nb:] == 0xA5).all()
+    return packed[:nb], sbf, mbf

@@ -7,6 +7,7 @@ GPU tests (-m gpu) remain the parity tests proper."""
 import numpy as np
 import pytest
 import scipy.sparse as sp
+import torch
 
 import emu_util as e
 import exact_oracle as o
@@ -199,3 +200,31 @@ def test_spmm_degenerate_row_layouts():
         got = e.spmm(rowptr, col, val, X, reduce, np.int32 if trial % 4 < 2 else np.int64)
         want = o.spmm_csr(rowptr, col, val, X, reduce)
         assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * max(1.0, np.abs(want).max())), (trial, M, N, K, mode)
+
+
+@pytest.mark.parametrize("N,G", [(203, 256), (64, 128), (37, 40), (19, 520), (16, 1024), (5, 8), (33, 100), (9, 1500)])
+def test_every_work_split_of_the_pack_kernel_gives_the_same_bytes(N, G):
+    """exact_minmax_pack_geom_f32: 1, 2 or 4 column groups per lane (and hints the
+    row length does not allow, which are ignored) -- identical results."""
+    rng = np.random.default_rng(N + G)
+    x = (rng.standard_normal((N, G)) * 2).astype(np.float32)
+    for bits in (1, 2, 4, 8):
+        want = o.quantize_activation(x, bits, o.philox_noise_rows(5, 9, N, G))
+        for hint in (0, 1, 2, 4):
+            if G > 1024:
+                continue                      # long rows need the fp32 outputs of the two-step form (covered elsewhere)
+            packed, sbf, mbf = e.minmax_pack_geom(x, bits, hint, None, 5, 9)
+            assert np.array_equal(packed, want[0]) and np.array_equal(sbf, want[2]) and np.array_equal(mbf, want[3]), (bits, hint)
+    assert e.minmax_pack_geom(x[:, :8], 2, 3, expect_rc=-5) is None
+
+
+def test_pack_geometry_candidates():
+    from exact_amd.cpp_extension import quantization as extq
+    assert extq.pack_geometry_candidates(256) == [1, 2, 4]
+    assert extq.pack_geometry_candidates(8) == [1]
+    assert extq.pack_geometry_candidates(16) == [1, 2]
+    assert extq.pack_geometry_candidates(520) == [4]          # 65 octs: only 4 per lane fits 32 lanes
+    assert extq.pack_geometry_candidates(1024) == [4]
+    assert extq.pack_geometry_candidates(2048) == []
+    t = torch.zeros(4, 256)
+    assert extq._pack_geometry(t, 2) == 0                      # host tensors (emulated runs) are never tuned

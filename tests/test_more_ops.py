@@ -415,3 +415,32 @@ def test_elu_backward_kernel(backend):
         assert got_h.dtype == torch.float16 and (got_h.float() - want_h.float()).abs().max() <= 2e-3 * want_h.float().abs().max()
     with pytest.raises(RuntimeError):
         bf._elu_backward_cuda(dy, x[:-1], 1.0)
+
+
+@pytest.mark.gpu
+def test_pack_work_split_is_tuned_once_and_never_changes_the_result(cuda):
+    """tune_pack_geometry times the 1 / 2 / 4 column-groups-per-lane forms of
+    the fused pack kernel; minmax_pack then uses the remembered one.  Whatever
+    it picks, the bytes are those of the oracle."""
+    from gpu_util import FixedNoise, bytes_equal, dev, host_noise, host_randn
+    N, G, bits = 8192, 256, 2
+    x = host_randn((N, G), 11)
+    u = host_noise((N, G), 12)
+    xt = dev(x)
+    extq._PACK_GEOMETRY.pop((G, bits), None)
+    timings = extq.tune_pack_geometry(xt, bits)
+    assert sorted(timings) == [1, 2, 4] and all(t > 0 for t in timings.values())
+    assert extq._PACK_GEOMETRY[(G, bits)] == min(timings, key=timings.get)
+    want = o.quantize_activation(x, bits, u)
+    for forced in (1, 2, 4):
+        extq._PACK_GEOMETRY[(G, bits)] = forced
+        config.noise_source = FixedNoise([dev(u)])
+        packed, sbf, mbf = extq.minmax_pack(xt, bits)
+        assert bytes_equal(packed, want[0]) and bytes_equal(sbf, want[2]) and bytes_equal(mbf, want[3])
+    extq._PACK_GEOMETRY.pop((G, bits), None)
+    config.noise_source = FixedNoise([dev(u)])
+    big = dev(host_randn((4096, 256), 13))                 # 2^20 elements: tuned on first use
+    extq._PACK_GEOMETRY.pop((256, 4), None)
+    config.noise_source = None
+    extq.minmax_pack(big, 4)
+    assert extq._PACK_GEOMETRY.get((256, 4)) in (1, 2, 4)
