@@ -309,12 +309,33 @@ def _extras_main(argv):
     print(json.dumps(run(x, log, budget_s=args.budget, scale=args.scale)), flush=True)
 
 
+def _epoch_main(argv):
+    """`python -m exact_amd.benchmarks epoch --config cfg3_gcn_int2 --epochs 5`:
+    a few full-batch training epochs of one model configuration, as the target
+    of a kernel trace (which kernels an epoch spends its time in)."""
+    import argparse
+    import json
+    ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks epoch")
+    ap.add_argument("--config", choices=sorted(EPOCH_CONFIGS), default="cfg3_gcn_int2")
+    ap.add_argument("--epochs", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--scale", type=float, default=1.0)
+    args = ap.parse_args(argv)
+
+    def log(*a):
+        print(*a, file=sys.stderr, flush=True)
+
+    res = epoch_benchmark(args.config, bench_device(), log, epochs=args.epochs, warmup=args.warmup, scale=args.scale)
+    print(json.dumps(res), flush=True)
+
+
 def _profile_target(argv=None):
     """One kernel in a loop, as the target of `rocprofv3 --kernel-trace --stats` /
     `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
 
         python -m exact_amd.benchmarks pack --bits 2 --reps 100
         python -m exact_amd.benchmarks {unpack,relu,dropout,rp_fwd,rp_bwd,spmm,copy} ...
+        python -m exact_amd.benchmarks epoch --config cfg3_gcn_int2 --epochs 5
 
     `copy` is a plain device-to-device copy of the same [rows, cols] fp32 tensor
     (4*rows*cols bytes read, as many written) for calibrating the byte counters."""
@@ -326,6 +347,8 @@ def _profile_target(argv=None):
         argv = sys.argv[1:]
     if argv and argv[0] == "extras":
         return _extras_main(argv[1:])
+    if argv and argv[0] == "epoch":
+        return _epoch_main(argv[1:])
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
     ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "rp_fwd", "rp_bwd", "spmm", "copy"])
     ap.add_argument("--bits", type=int, default=2)

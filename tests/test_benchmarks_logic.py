@@ -121,3 +121,11 @@ def test_failed_extras_child_leaves_an_error_entry(monkeypatch):
         raise subprocess.TimeoutExpired(a[0], 1)
     monkeypatch.setattr(subprocess, "run", boom)
     assert "exceeded" in bench.run_extras(10, 8, 1.0)["error"]
+
+
+def test_epoch_entry_point(cpu_harness, capsys):
+    """`python -m exact_amd.benchmarks epoch` (the target of a kernel trace of one model configuration)."""
+    import json
+    bm._profile_target(["epoch", "--config", "cfg3_gcn_int2", "--epochs", "1", "--warmup", "0", "--scale", "0.0005"])
+    res = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert res["epochs_per_s"] > 0 and res["bits"] == 2
