@@ -51,6 +51,10 @@ _EXTRA_FIELDS = {
     # groups per lane) the first time a large activation of a new (width, bits)
     # is compressed on a GPU, and keep the fastest.  Results do not depend on it.
     "autotune_pack": True,
+    # Sparse products with a reproducible (CSR-order, atomics-free) summation;
+    # also switched on by torch.use_deterministic_algorithms(True).  The default
+    # kernel balances hub rows across wavefronts and adds their parts atomically.
+    "deterministic_spmm": False,
 }
 
 

@@ -9,6 +9,7 @@ from collections import OrderedDict
 import torch
 
 from .. import _lib
+from ..conf import config
 from . import _checks
 from ._checks import ptr
 
@@ -55,8 +56,10 @@ def spmm_csr(rowptr, col, value, mat, reduce):
     M = rowptr.numel() - 1
     n_cols, K = mat.shape
     out = torch.empty((M, K), dtype=mat.dtype, device=mat.device)
-    rc = _lib.lib().exact_spmm_csr_f32(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat),
-                                       M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out), _checks.stream_ptr(mat))
+    reproducible = config.deterministic_spmm or torch.are_deterministic_algorithms_enabled()
+    kernel = _lib.lib().exact_spmm_csr_rowwise_f32 if reproducible else _lib.lib().exact_spmm_csr_f32
+    rc = kernel(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat),
+                M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out), _checks.stream_ptr(mat))
     _lib.check(rc, f"spmm_{reduce}")
     return out
 

@@ -62,6 +62,46 @@ __global__ __launch_bounds__(kBlock) void spmm_minmax_kernel(const I* __restrict
   }
 }
 
+// Deterministic sum / mean: one wavefront per row (and per slab of 64 * VEC
+// columns), the row's entries taken one after the other in CSR order with one
+// multiply and one add each -- the summation order of the reference kernel
+// (spmm_cuda.cu:85-90) and of the CPU oracle, so results are reproducible bit
+// for bit.  No atomics, every output element is stored exactly once.  Hub rows
+// serialise, which is why the default path is the chunked kernel in spmm.hip.
+template <typename I, int VEC, bool HAS_VAL, bool MEAN>
+__global__ __launch_bounds__(kBlock) void spmm_rowwise_kernel(const I* __restrict__ rowptr,
+                                                              const I* __restrict__ col,
+                                                              const float* __restrict__ val,
+                                                              const float* __restrict__ X, int64_t M, int64_t K,
+                                                              float* __restrict__ out) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t r = static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + (threadIdx.x >> 6);
+  if (r >= M) return;
+  const int64_t kcol = (static_cast<int64_t>(blockIdx.y) * kWave + lane) * VEC;
+  if (kcol >= K) return;
+  const int64_t rs = static_cast<int64_t>(rowptr[r]), re = static_cast<int64_t>(rowptr[r + 1]);
+  float acc[VEC];
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) acc[c] = 0.f;
+  for (int64_t e = rs; e < re; ++e) {
+    float xv[VEC];
+    load_cols<VEC>(X + static_cast<int64_t>(col[e]) * K + kcol, xv);
+    const float w = HAS_VAL ? val[e] : 1.f;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+      const float term = HAS_VAL ? w * xv[c] : xv[c];
+      acc[c] = acc[c] + term;
+    }
+  }
+  if (MEAN) {
+    const float cnt = static_cast<float>(re > rs ? re - rs : 1);  // reducer.cuh:75-76
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) acc[c] = acc[c] / cnt;
+  }
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) out[r * K + kcol + c] = acc[c];
+}
+
 // out[e] = sum_k mat[col[e], k] * grad[row[e], k]   (/ max(deg(row[e]), 1) for mean)
 template <typename I, int VEC, bool MEAN>
 __global__ __launch_bounds__(kBlock) void sddmm_kernel(const I* __restrict__ row, const I* __restrict__ rowptr,
@@ -116,6 +156,20 @@ static void sddmm_dispatch(const I* row, const I* rowptr, const I* col, const fl
   else hipLaunchKernelGGL((sddmm_kernel<I, VEC, false>), grid, dim3(kBlock), 0, s, row, rowptr, col, mat, grad, E, K, out);
 }
 
+template <typename I, int VEC>
+static void rowwise_dispatch(const I* rowptr, const I* col, const float* val, const float* X, int64_t M, int64_t K,
+                             bool mean, float* out, hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>((M + 3) / 4), static_cast<unsigned>((K + kWave * VEC - 1) / (kWave * VEC)));
+  const dim3 block(kBlock);
+  if (val) {
+    if (mean) hipLaunchKernelGGL((spmm_rowwise_kernel<I, VEC, true, true>), grid, block, 0, s, rowptr, col, val, X, M, K, out);
+    else hipLaunchKernelGGL((spmm_rowwise_kernel<I, VEC, true, false>), grid, block, 0, s, rowptr, col, val, X, M, K, out);
+  } else {
+    if (mean) hipLaunchKernelGGL((spmm_rowwise_kernel<I, VEC, false, true>), grid, block, 0, s, rowptr, col, val, X, M, K, out);
+    else hipLaunchKernelGGL((spmm_rowwise_kernel<I, VEC, false, false>), grid, block, 0, s, rowptr, col, val, X, M, K, out);
+  }
+}
+
 }  // namespace exact
 
 using namespace exact;
@@ -163,6 +217,30 @@ int exact_sddmm_f32(const void* row, const void* rowptr, const void* col, int id
     if (vec == 4) EXACT_SD_GO(int64_t, 4); else if (vec == 2) EXACT_SD_GO(int64_t, 2); else EXACT_SD_GO(int64_t, 1);
   }
 #undef EXACT_SD_GO
+  return launch_status();
+}
+
+int exact_spmm_csr_rowwise_f32(const void* rowptr, const void* col, const float* val, int idx_bytes, const float* X,
+                               int64_t M, int64_t n_cols, int64_t K, int64_t nnz, int reduce, float* out,
+                               void* stream) {
+  if (idx_bytes != 4 && idx_bytes != 8) return EXACT_E_ARG;
+  if (reduce != EXACT_REDUCE_SUM && reduce != EXACT_REDUCE_MEAN) return EXACT_E_ARG;
+  if (M < 0 || K < 0 || nnz < 0 || n_cols < 0 || n_cols > 0x7FFFFFFFll) return EXACT_E_SHAPE;
+  if (idx_bytes == 4 && nnz > 0x7FFFFFFFll) return EXACT_E_SHAPE;
+  if (M > (int64_t{1} << 32) || K > (int64_t{1} << 24)) return EXACT_E_SHAPE;  // launch-grid limits
+  if (M == 0 || K == 0) return EXACT_OK;
+  if (!rowptr || !out || (nnz > 0 && (!col || !X))) return EXACT_E_NULL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool mean = reduce == EXACT_REDUCE_MEAN;
+  const int vec = (K % 4 == 0 && aligned_to(X, 16)) ? 4 : (K % 2 == 0 && aligned_to(X, 8)) ? 2 : 1;
+#define EXACT_RW_GO(I, V) \
+  rowwise_dispatch<I, V>(static_cast<const I*>(rowptr), static_cast<const I*>(col), val, X, M, K, mean, out, s)
+  if (idx_bytes == 4) {
+    if (vec == 4) EXACT_RW_GO(int32_t, 4); else if (vec == 2) EXACT_RW_GO(int32_t, 2); else EXACT_RW_GO(int32_t, 1);
+  } else {
+    if (vec == 4) EXACT_RW_GO(int64_t, 4); else if (vec == 2) EXACT_RW_GO(int64_t, 2); else EXACT_RW_GO(int64_t, 1);
+  }
+#undef EXACT_RW_GO
   return launch_status();
 }
 

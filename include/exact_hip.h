@@ -133,6 +133,13 @@ int exact_spmm_csr_f32(const void *rowptr, const void *col, const float *val,
                        int idx_bytes, const float *X, int64_t M, int64_t n_cols,
                        int64_t K, int64_t nnz, int reduce, float *out, void *stream);
 
+/* The same product with a reproducible result: one wavefront per row, entries
+ * added in CSR order with one multiply and one add each (the order of the
+ * reference kernel, spmm_cuda.cu:85-90), no atomics.  Slower on hub rows. */
+int exact_spmm_csr_rowwise_f32(const void *rowptr, const void *col, const float *val,
+                               int idx_bytes, const float *X, int64_t M, int64_t n_cols,
+                               int64_t K, int64_t nnz, int reduce, float *out, void *stream);
+
 /* Max / min aggregation: out[r, k] = max (is_max != 0) or min over the entries
  * e of row r of val[e] * X[col[e], k]; arg_out[r, k] (same index type as
  * rowptr / col, [M, K]) = the first entry index attaining it; rows without

@@ -162,6 +162,10 @@ static void check_spmm(int64_t M, int64_t ncols, int64_t K, double avg, int64_t 
         for (int64_t i = 0; i < M * K; ++i) scale = std::max(scale, (double)std::fabs(want[i]));
         for (int64_t i = 0; i < M * K; ++i) worst = std::max(worst, (double)std::fabs(out[i] - want[i]));
         CHECK(worst <= 1e-5 * scale, "spmm differs M=%ld K=%ld reduce=%d valued=%d wide=%d: %g of %g", (long)M, (long)K, reduce, valued, wide, worst, scale);
+        // the reproducible kernel sums in the oracle's order: bit-identical
+        const int rc2 = wide ? exact_spmm_csr_rowwise_f32(rp64.p, col64.p, valued ? val.p : nullptr, 8, X.p, M, ncols, K, nnz, reduce, out.p, nullptr)
+                             : exact_spmm_csr_rowwise_f32(rp32.p, col32.p, valued ? val.p : nullptr, 4, X.p, M, ncols, K, nnz, reduce, out.p, nullptr);
+        CHECK(rc2 == 0 && std::memcmp(out.p, want.p, M * K * 4) == 0, "rowwise spmm differs M=%ld K=%ld reduce=%d valued=%d wide=%d", (long)M, (long)K, reduce, valued, wide);
       }
 }
 

@@ -330,3 +330,17 @@ def minmax_pack_geom(x, bits, octs_per_lane, noise=None, seed=0, offset=0, guard
         return None
     assert (packed[nb:] == 0xA5).all()
     return packed[:nb], sbf, mbf
+
+
+def spmm_rowwise(rowptr, col, val, X, reduce, idx=np.int64, guard=16):
+    rowptr = np.ascontiguousarray(rowptr, dtype=idx)
+    col = np.ascontiguousarray(col, dtype=idx)
+    X = f32(X)
+    val = None if val is None else f32(val)
+    M, K = rowptr.size - 1, X.shape[1]
+    out = np.full(M * K + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_spmm_csr_rowwise_f32(p(rowptr), p(col), p(val), rowptr.itemsize, p(X), M, X.shape[0], K, col.size,
+                                          1 if reduce == "mean" else 0, p(out), None)
+    assert rc == 0, rc
+    assert (out[M * K:] == np.float32(-777.0)).all()
+    return out[:M * K].reshape(M, K)

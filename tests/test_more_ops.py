@@ -444,3 +444,47 @@ def test_pack_work_split_is_tuned_once_and_never_changes_the_result(cuda):
     config.noise_source = None
     extq.minmax_pack(big, 4)
     assert extq._PACK_GEOMETRY.get((256, 4)) in (1, 2, 4)
+
+
+@pytest.mark.parametrize("idx", [np.int64, np.int32])
+@pytest.mark.parametrize("valued", [True, False])
+@pytest.mark.parametrize("reduce", ["sum", "mean"])
+@pytest.mark.parametrize("M,N,K", [(60, 40, 256), (33, 50, 40), (20, 20, 602), (45, 30, 7), (9, 12, 1), (300, 100, 100)])
+def test_rowwise_spmm_kernel_is_bit_identical_to_the_oracle(M, N, K, reduce, valued, idx):
+    """The reproducible kernel sums in CSR order with one multiply and one add
+    per entry -- exactly what the oracle (and its C twin) do."""
+    import c_oracle as co
+    A = csr(M, N, M * 7, M + K)
+    X = np.random.default_rng(K).standard_normal((N, K)).astype(F32)
+    val = A.data if valued else None
+    got = e.spmm_rowwise(A.indptr, A.indices, val, X, reduce, idx)
+    want = o.spmm_csr(A.indptr, A.indices, val, X, reduce)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(co.spmm_csr(A.indptr, A.indices, val, X, reduce).view(np.uint32), want.view(np.uint32))
+
+
+def test_deterministic_spmm_switch(backend):
+    """config.deterministic_spmm / torch.use_deterministic_algorithms select the
+    reproducible kernel for forward and backward; the result is the oracle's, bit for bit."""
+    A = csr(400, 400, 6000, 3, empty_rows=True)
+    g = torch.Generator().manual_seed(5)
+    X, dY = torch.randn(400, 64, generator=g), torch.randn(400, 64, generator=g)
+    adj = SparseTensor.from_scipy(A, backend)
+    want = o.spmm_csr(A.indptr, A.indices, A.data, X.numpy(), "sum")
+    At = A.T.tocsr()
+    At.sort_indices()
+    want_bw = o.spmm_csr(At.indptr, At.indices, At.data, dY.numpy(), "sum")
+    for how in ("config", "torch"):
+        if how == "config":
+            config.deterministic_spmm = True
+        else:
+            config.deterministic_spmm = False
+            torch.use_deterministic_algorithms(True)
+        try:
+            x = X.clone().to(backend).requires_grad_()
+            y = qmatmul(adj, x, "sum")
+            y.backward(dY.to(backend))
+        finally:
+            torch.use_deterministic_algorithms(False)
+        assert np.array_equal(y.detach().cpu().numpy().view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(x.grad.cpu().numpy().view(np.uint32), want_bw.view(np.uint32))
