@@ -38,7 +38,8 @@ def build_asan_check():
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
     oracle_o = os.path.join(OUT, "exact_oracle.o")
     _run(["gcc", "-O2", "-ffp-contract=off", "-c", os.path.join(ROOT, "oracle", "exact_oracle.c"), "-o", oracle_o])
-    _run([CLANG, *COMMON, "-O1", "-g", "-fsanitize=address", "-fno-omit-frame-pointer", "-o", CHECK,
+    _run([CLANG, *COMMON, "-O1", "-g", "-fsanitize=address,alignment,bounds,shift", "-fno-sanitize-recover=alignment,bounds,shift",
+          "-fno-omit-frame-pointer", "-o", CHECK,
           *srcs, "-x", "c++", os.path.join(HERE, "emu_check.cpp"), "-x", "none", oracle_o, "-lm"])
     return CHECK
 
