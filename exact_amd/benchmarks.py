@@ -125,6 +125,15 @@ def kernel_extras(x, log):
             t_pack = event_time(lambda: extq.minmax_pack(x, 2))
             out["relu_dropout_pack_int2"] = {"us": t * 1e6, "GB/s": fused_bytes / t / 1e9, "algo_bytes": fused_bytes,
                                              "replaces_us": out["relu_fwd"]["us"] + out["dropout_fwd"]["us"] + t_pack * 1e6}
+            # batch norm folded in: statistics (torch.var_mean) + the one pass, against
+            # native_batch_norm + the ReLU / dropout / pack pass
+            col = torch.ones(G, device=x.device)
+            t_fold = event_time(lambda: extq.bn_relu_dropout_minmax_pack(x, col, col, col, 0.5, 2))
+            t_stats = event_time(lambda: torch.var_mean(x, dim=0, unbiased=False))
+            t_bn = event_time(lambda: torch.ops.aten.native_batch_norm(x, col, col, None, None, True, 0.1, 1e-5))
+            out["bn_relu_dropout_pack_int2"] = {"us": t_fold * 1e6, "GB/s": fused_bytes / t_fold / 1e9,
+                                                "algo_bytes": fused_bytes, "stats_us": t_stats * 1e6,
+                                                "replaces_us": t_bn * 1e6 + t * 1e6}
         # --- random projection 256 -> 32 (kept_frac 0.125), Gaussian N(0, 1/k) --
         k = int(0.125 * G + 0.999)
         R = torch.randn(G, k, device=x.device) / k ** 0.5

@@ -47,6 +47,11 @@ _EXTRA_FIELDS = {
     # model offers the pair as one module (QReLUDropout).  Results are
     # bit-identical to the separate layers; False runs them separately.
     "fuse_epilogue": True,
+    # A QBatchNorm1d ahead of that pair joins the same pass (normalise -> ReLU ->
+    # dropout -> quantise).  The batch statistics then come from torch.var_mean
+    # instead of native_batch_norm, so results agree with the separate layers to
+    # rounding (about 1e-6 relative), not bit for bit.  Needs fuse_epilogue.
+    "fold_batch_norm": True,
     # Time the alternative work splits of the pack kernel (1, 2 or 4 column
     # groups per lane) the first time a large activation of a new (width, bits)
     # is compressed on a GPU, and keep the fastest.  Results do not depend on it.

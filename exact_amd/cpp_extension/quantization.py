@@ -344,6 +344,35 @@ def relu_dropout_minmax_pack(input, p, bits):  # noqa: A002
     return out, mask, packed, scale_bf, min_bf
 
 
+def bn_relu_dropout_minmax_pack(input, mean, mult, shift, p, bits):  # noqa: A002
+    """relu_dropout_minmax_pack of the batch-normalised input, (input - mean) *
+    mult + shift per column (three fp32 operations), in the same single pass
+    -> (output, mask, packed int8, scale bf16, min bf16)."""
+    check_device_tensor(input, "input", 2)
+    _check_bits(bits)
+    N, G = input.shape
+    for name, vec in (("mean", mean), ("mult", mult), ("shift", shift)):
+        check_device_tensor(vec, name, 1)
+        if vec.shape[0] != G:
+            raise RuntimeError(f"The dimension of {name} is not correct!")
+    if not fusable_width(G):
+        raise RuntimeError("bn_relu_dropout_minmax_pack needs a row width that is a multiple of 8 and at most 1024")
+    dev = input.device
+    out = torch.empty_like(input)
+    mask = torch.empty(mask_nwords(N * G), dtype=torch.int32, device=dev)
+    packed = torch.empty(packed_nbytes(N, G, bits), dtype=torch.int8, device=dev)
+    scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    act_noise, act_seed, act_offset = _noise_for(input.shape, dev)
+    noise, seed, offset = _noise_for(input.shape, dev)
+    rc = _lib.lib().exact_bn_relu_dropout_minmax_pack_f32(
+        ptr(input), ptr(mean), ptr(mult), ptr(shift), float(p), ptr(act_noise), act_seed, act_offset, ptr(noise), seed,
+        offset, N, G, bits, ptr(out), ptr(mask), ptr(packed), None, None, ptr(scale_bf), ptr(min_bf),
+        _checks.stream_ptr(input))
+    _lib.check(rc, "bn_relu_dropout_minmax_pack")
+    return out, mask, packed, scale_bf, min_bf
+
+
 def dropout_bwd(grad_output, mask, p):
     """dx = bit ? dy / (1 - p) : 0 (quantization_cuda_kernel.cu:565-569)."""
     grad_output = grad_output.contiguous()

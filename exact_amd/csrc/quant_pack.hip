@@ -70,6 +70,15 @@ __device__ __forceinline__ void load_oct_half(const half_t* __restrict__ p, int 
   }
 }
 
+// 8 consecutive floats that every workgroup reads again (per-column
+// parameters): ordinary cached loads, 16-byte aligned
+__device__ __forceinline__ void load_cached8(const float* __restrict__ p, float (&v)[8]) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p);
+  const f32x4 b = *reinterpret_cast<const f32x4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
 // ---------------------------------------------------------------------------
 // pack
 // ---------------------------------------------------------------------------
@@ -97,6 +106,10 @@ struct PackArgs {
   float* y;                // activation output [N, G]
   uint8_t* mask_bytes;     // 1-bit mask of (x > 0) && keep, byte i / 8 holds elements i .. i + 7
   int64_t mask_tail_begin, mask_tail_end;  // bytes of the last mask word no element maps to
+  // ACT form, optional: per-column normalisation (x - mean) * mult + shift ahead of the ReLU
+  const float* norm_mean;   // nullable: no normalisation
+  const float* norm_mult;
+  const float* norm_shift;
 };
 
 // ACT: x first goes through ReLU and dropout (the arithmetic of
@@ -154,6 +167,20 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
           const Philox4 r = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32),
                                           a.act_off_lo, a.act_off_hi, a.act_seed_lo, a.act_seed_hi);
           philox_uniform8(r, ud);
+        }
+        if (a.norm_mean != nullptr) {  // same for every lane of the launch
+          // training-mode batch norm of the column, statistics given:
+          // weight * (x - mean) * invstd + bias with mult = weight * invstd
+          float cm[8], cs[8], cb[8];
+          load_cached8(a.norm_mean + d0, cm);
+          load_cached8(a.norm_mult + d0, cs);
+          load_cached8(a.norm_shift + d0, cb);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            float c = v[k][i] - cm[i];
+            c = c * cs[i];
+            v[k][i] = c + cb[i];
+          }
         }
         uint32_t m = 0;
 #pragma unroll
@@ -600,11 +627,12 @@ int exact_minmax_pack_geom_f32(const float* x, const float* noise, uint64_t seed
                      scale_bf16, min_bf16, true, static_cast<hipStream_t>(stream), octs_per_lane);
 }
 
-int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act_noise, uint64_t act_seed,
-                                       uint64_t act_offset, const float* noise, uint64_t seed, uint64_t offset,
-                                       int64_t N, int64_t G, int bits, float* y, uint32_t* mask, uint8_t* packed,
-                                       float* scale_f32, float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16,
-                                       void* stream) {
+static int act_pack_common(const float* x, const float* norm_mean, const float* norm_mult,
+                           const float* norm_shift, float p, const float* act_noise, uint64_t act_seed,
+                           uint64_t act_offset, const float* noise, uint64_t seed, uint64_t offset,
+                           int64_t N, int64_t G, int bits, float* y, uint32_t* mask, uint8_t* packed,
+                           float* scale_f32, float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16,
+                           void* stream) {
   if (int rc = check_quant_shape(N, G, bits)) return rc;
   if (!(p >= 0.f && p < 1.f)) return EXACT_E_ARG;
   if ((act_noise == nullptr) != (noise == nullptr)) return EXACT_E_ARG;  // both streams supplied, or neither
@@ -619,9 +647,14 @@ int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act
   if (!x || !y || !mask) return EXACT_E_NULL;
   if (!aligned(x, 16) || !aligned(y, 16) || (noise && (!aligned(noise, 16) || !aligned(act_noise, 16))))
     return EXACT_E_ALIGN;
+  if (norm_mean && (!aligned(norm_mean, 16) || !aligned(norm_mult, 16) || !aligned(norm_shift, 16)))
+    return EXACT_E_ALIGN;
   const Geometry g = plan_rows(G, 4);
   PackArgs a{};
   a.x = x;
+  a.norm_mean = norm_mean;
+  a.norm_mult = norm_mult;
+  a.norm_shift = norm_shift;
   a.noise = noise;
   a.mn_in = nullptr;
   a.scale_in = nullptr;
@@ -657,6 +690,25 @@ int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act
   if (noise) launch_act_bits<true>(a, bits, g.opt, g.full, grid, s);
   else launch_act_bits<false>(a, bits, g.opt, g.full, grid, s);
   return launch_status();
+}
+
+int exact_relu_dropout_minmax_pack_f32(const float* x, float p, const float* act_noise, uint64_t act_seed,
+                                       uint64_t act_offset, const float* noise, uint64_t seed, uint64_t offset,
+                                       int64_t N, int64_t G, int bits, float* y, uint32_t* mask, uint8_t* packed,
+                                       float* scale_f32, float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16,
+                                       void* stream) {
+  return act_pack_common(x, nullptr, nullptr, nullptr, p, act_noise, act_seed, act_offset, noise, seed, offset, N, G,
+                         bits, y, mask, packed, scale_f32, min_f32, scale_bf16, min_bf16, stream);
+}
+
+int exact_bn_relu_dropout_minmax_pack_f32(const float* x, const float* mean, const float* mult, const float* shift,
+                                          float p, const float* act_noise, uint64_t act_seed, uint64_t act_offset,
+                                          const float* noise, uint64_t seed, uint64_t offset, int64_t N, int64_t G,
+                                          int bits, float* y, uint32_t* mask, uint8_t* packed, float* scale_f32,
+                                          float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, void* stream) {
+  if (N > 0 && G > 0 && (!mean || !mult || !shift)) return EXACT_E_NULL;
+  return act_pack_common(x, mean, mult, shift, p, act_noise, act_seed, act_offset, noise, seed, offset, N, G, bits, y,
+                         mask, packed, scale_f32, min_f32, scale_bf16, min_bf16, stream);
 }
 
 int exact_minmax_pack_f16(const uint16_t* x, const float* noise, uint64_t seed, uint64_t offset, int64_t N,

@@ -15,8 +15,8 @@ from torch.nn import Parameter
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCN2Conv, GCNConv, GENConv, GraphConv, SAGEConv, glorot
-from .ops import (input2rp, kept_columns, qbatch_norm, qelu, qlinear, quantize_activation, relu_dropout,
-                  take_compressed)
+from .ops import (bn_relu_dropout, consumer_bits, input2rp, kept_columns, qbatch_norm, qelu, qlinear,
+                  quantize_activation, relu_dropout, take_compressed)
 from .qsheme import QScheme
 from .spmm import QMatmul, qmatmul
 
@@ -269,6 +269,26 @@ class QReLUDropout(_TrainEval):
         super().__init__()
         self.p = p
         self.for_consumer = for_consumer
+
+    def forward(self, input, norm=None):  # noqa: A002
+        """`norm`: a batch norm layer to apply ahead of the ReLU; a QBatchNorm1d in
+        training mode is folded into the same pass where the kernel applies."""
+        if norm is not None:
+            fused = self._with_norm(input, norm) if self.training else None
+            if fused is not None:
+                return fused
+            input = norm(input)  # noqa: A001
+        return super().forward(input)
+
+    def _with_norm(self, t, norm):
+        if not (isinstance(norm, QBatchNorm1d) and norm.training and config.fuse_epilogue and config.fold_batch_norm
+                and t.dim() == 2):
+            return None
+        bits = consumer_bits(t, self.for_consumer)
+        if bits is None or t.shape[0] < 2:
+            return None                      # not this kernel's case
+        norm._check_input_dim(t)
+        return bn_relu_dropout(t, norm, norm._averaging_factor(), self.p, bits)
 
     def _train(self, t):
         return relu_dropout(t, self.p, self.for_consumer)

@@ -38,11 +38,13 @@ class _Stack(torch.nn.Module):
             x = self.input_dropout(x)
         for idx, conv in enumerate(self.convs[:-1]):
             h = conv(x, adj_t)
-            if self.batch_norm:
-                h = self.bns[idx](h)
+            norm = self.bns[idx] if self.batch_norm else None
             if self.residual and h.size(-1) == x.size(-1):
-                h = h + x[:h.size(0)]
-            x = self.act_drop(h)
+                if norm is not None:
+                    h = norm(h)
+                x = self.act_drop(h + x[:h.size(0)])
+            else:
+                x = self.act_drop(h, norm=norm)    # norm -> ReLU -> dropout as one unit (one pass when quantised)
         return self.convs[-1](x, adj_t)
 
 

@@ -35,10 +35,17 @@ def _dropout(p):
     return QDropout2(p) if config.dropout2 else QDropout(p)        # module.py:38-42
 
 
+class _ReLUThenDropout(nn.Sequential):
+    """The two quantised layers one after the other, callable like ReLUDropout."""
+
+    def forward(self, input, norm=None):  # noqa: A002
+        return super().forward(input if norm is None else norm(input))
+
+
 def _relu_dropout(src):
     if config.fuse_epilogue and not config.dropout2:
         return QReLUDropout(src.p)
-    return nn.Sequential(QReLU(), _dropout(src.p))
+    return _ReLUThenDropout(QReLU(), _dropout(src.p))
 
 
 def _gcn2(src):                                                      # module.py:47-53

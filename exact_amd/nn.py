@@ -138,7 +138,11 @@ class ReLUDropout(torch.nn.Module):
         super().__init__()
         self.p = p
 
-    def forward(self, input):  # noqa: A002
+    def forward(self, input, norm=None):  # noqa: A002
+        """`norm`: a normalisation layer to apply first (the quantised counterpart
+        folds a batch norm into its pass)."""
+        if norm is not None:
+            input = norm(input)  # noqa: A001
         return F.dropout(F.relu(input), self.p, self.training)
 
     def extra_repr(self):

@@ -459,6 +459,52 @@ class qrelu_dropout(Function):
         return ext_quantization.dropout_bwd(grad_output, mask, ctx.p), None, None
 
 
+class qbn_relu_dropout(Function):
+    """Training-mode batch norm -> ReLU -> dropout, the chain QBatchNorm1d ->
+    QReLU -> QDropout of the reference (layers.py:340-369, 284-325; ops.py:206-254),
+    in two passes over the input instead of six: the batch norm's compressed
+    copy of its input (ops.py:213), the batch statistics, and then ONE pass that
+    normalises, applies ReLU and dropout with one joint mask and quantises the
+    result for the following layer.  Backward: the joint mask, then
+    native_batch_norm_backward on the dequantised input as in ops.py:228-254.
+    -> (output, packed, scale bf16, min bf16)."""
+
+    @staticmethod
+    def forward(ctx, input, running_mean, running_var, weight, bias,  # noqa: A002
+                exponential_average_factor, eps, p, bits, scheme):
+        kept = CompressedActivation.compress(input, scheme, project=False)
+        rows = input.shape[0]
+        var, mean = torch.var_mean(input, dim=0, unbiased=False)
+        invstd = torch.rsqrt(var + eps)
+        if running_mean is not None:                       # the bookkeeping of native_batch_norm
+            running_mean.mul_(1 - exponential_average_factor).add_(mean, alpha=exponential_average_factor)
+            running_var.mul_(1 - exponential_average_factor).add_(var * (rows / max(rows - 1, 1)),
+                                                                   alpha=exponential_average_factor)
+        mult = invstd if weight is None else weight * invstd
+        shift = torch.zeros_like(mean) if bias is None else bias.detach()
+        out, mask, packed, scale, mn = ext_quantization.bn_relu_dropout_minmax_pack(
+            input, mean, mult.contiguous(), shift.contiguous(), p, bits)
+        ctx.mark_non_differentiable(packed, scale, mn)
+        ctx.save_for_backward(mask)
+        ctx.kept = kept
+        ctx.stats = (weight, running_mean, running_var, mean, invstd, eps)
+        ctx.p = float(p)
+        return out, packed, scale, mn
+
+    @staticmethod
+    def backward(ctx, grad_output, *unused):
+        (mask,) = ctx.saved_tensors
+        weight, running_mean, running_var, save_mean, save_invstd, eps = ctx.stats
+        grad_normalised = ext_quantization.dropout_bwd(grad_output, mask, ctx.p)
+        x_hat = ctx.kept.restore()
+        ctx.kept = None
+        empty_cache(config.empty_cache_threshold)
+        wanted = [ctx.needs_input_grad[0], ctx.needs_input_grad[3], ctx.needs_input_grad[4]]
+        g_in, g_w, g_b = ext_backward_func.native_batch_norm_backward(
+            grad_normalised, x_hat, weight, running_mean, running_var, save_mean, save_invstd, True, eps, wanted)
+        return g_in, None, None, g_w, g_b, None, None, None, None, None
+
+
 # Compressed copies made ahead of their consumer, keyed by the tensor they
 # describe.  The entry dies with the tensor; `_version` guards against an
 # in-place change between producer and consumer.
@@ -482,17 +528,38 @@ def take_compressed(tensor, project=True):
     return quantized if usable else None
 
 
+def consumer_bits(input, for_consumer):  # noqa: A002
+    """Bit width of the compressed copy the fused pass can make of its result for
+    the next layer, or None where it cannot (needs 2-D fp32 rows of a multiple
+    of 8 <= 1024 columns, compression on, no projection, no autocast)."""
+    if (for_consumer and config.compress_activation and config.kept_frac == 1.0 and input.dim() == 2
+            and input.dtype == torch.float32 and not torch.is_autocast_enabled()
+            and not config.simulate and ext_quantization.fusable_width(input.shape[1])):
+        return config.activation_compression_bits[0]
+    return None
+
+
+def bn_relu_dropout(input, norm, exponential_average_factor, p, bits):  # noqa: A002
+    """dropout(relu(batch_norm(input))) in training mode through qbn_relu_dropout;
+    `bits` from consumer_bits(input, True) (not None), at least two rows.
+    `norm` supplies running statistics, affine parameters, eps and scheme of a
+    QBatchNorm1d; the compressed copy of the result is handed over to the layer
+    that receives it."""
+    check_device_tensor(input, "input", 2)
+    running = (norm.running_mean, norm.running_var) if norm.track_running_stats else (None, None)
+    out, packed, scale, mn = qbn_relu_dropout.apply(input, *running, norm.weight, norm.bias,
+                                                    exponential_average_factor, norm.eps, p, bits, norm.scheme)
+    hand_over_compressed(out, (swap_to_cpu(packed) if config.swap else packed, bits, scale, mn))
+    return out
+
+
 def relu_dropout(input, p, for_consumer=False):  # noqa: A002
     """dropout(relu(input)); with `for_consumer`, the compressed copy of the
     result is made in the same pass where the kernel can (2-D rows of a
     multiple of 8 <= 1024 columns, compression on, no projection) and handed
     over to the layer that receives the result."""
     check_device_tensor(input, "input", None, FLOAT_OR_HALF)
-    bits = None
-    if (for_consumer and config.compress_activation and config.kept_frac == 1.0 and input.dim() == 2
-            and input.dtype == torch.float32 and not torch.is_autocast_enabled()
-            and not config.simulate and ext_quantization.fusable_width(input.shape[1])):
-        bits = config.activation_compression_bits[0]
+    bits = consumer_bits(input, for_consumer)
     out, packed, scale, mn = qrelu_dropout.apply(input, p, bits)
     if bits is not None:
         hand_over_compressed(out, (swap_to_cpu(packed) if config.swap else packed, bits, scale, mn))

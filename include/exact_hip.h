@@ -203,6 +203,22 @@ int exact_relu_dropout_minmax_pack_f32(const float *x, float p, const float *act
                                        float *min_f32, uint16_t *scale_bf16,
                                        uint16_t *min_bf16, void *stream);
 
+/* The same pass with training-mode batch norm ahead of the ReLU: every element
+ * of column c first becomes (x - mean[c]) * mult[c] + shift[c] (three separate
+ * fp32 operations), i.e. native_batch_norm's weight * (x - mean) * invstd + bias
+ * (layers.py:340-369, ops.py:206-225) with mult = weight * invstd and the batch
+ * statistics supplied by the caller; then ReLU, dropout, mask and the packed
+ * copy of the result exactly as exact_relu_dropout_minmax_pack_f32.  mean,
+ * mult and shift are fp32[G], 16-byte aligned.  Same shape conditions. */
+int exact_bn_relu_dropout_minmax_pack_f32(const float *x, const float *mean, const float *mult,
+                                          const float *shift, float p, const float *act_noise,
+                                          uint64_t act_seed, uint64_t act_offset,
+                                          const float *noise, uint64_t seed, uint64_t offset,
+                                          int64_t N, int64_t G, int bits, float *y,
+                                          uint32_t *mask, uint8_t *packed, float *scale_f32,
+                                          float *min_f32, uint16_t *scale_bf16,
+                                          uint16_t *min_bf16, void *stream);
+
 /* fp16 activations (row f4: the reference instantiates its kernels for
  * at::Half as well -- AT_DISPATCH_FLOATING_TYPES_AND_HALF at
  * quantization_cuda_kernel.cu:132-150, 209-226, 284, 324, 387, 428, 535, 586 --

@@ -307,6 +307,30 @@ static void check_fused(int64_t N, int64_t G, int bits, bool supplied, std::mt19
   CHECK(rc == 0 && std::memcmp(y.p, y2.p, n * 4) == 0 && bad == 0, "fused y/mask differ N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
   CHECK(std::memcmp(packed.p, want.p, nb) == 0, "fused packed differs N=%ld G=%ld bits=%d supplied=%d", (long)N, (long)G, bits, supplied);
   CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "fused scale/min differ N=%ld G=%ld", (long)N, (long)G);
+  // with batch norm ahead: the same chain on (x - mean) * mult + shift, three roundings
+  Buf<float> mean(G), mult(G), shift(G), xn(n);
+  for (int64_t d = 0; d < G; ++d) { mean[d] = nd(rng); mult[d] = 0.5f + ud(rng); shift[d] = 0.25f * nd(rng); }
+  for (int64_t i = 0; i < n; ++i) {
+    volatile float c = x[i] - mean[i % G];
+    c = c * mult[i % G];
+    xn[i] = c + shift[i % G];
+  }
+  oracle_relu_fwd(xn.p, n, y1.p, m1.p);
+  oracle_dropout_fwd(y1.p, supplied ? ua.p : nullptr, s1, o1, p, n, y2.p, m2.p);
+  oracle_row_minmax(y2.p, N, G, mn.p, mx.p);
+  oracle_scale(mn.p, mx.p, N, bits, sc.p);
+  std::memset(want.p, 0, nb);
+  oracle_pack(y2.p, mn.p, sc.p, supplied ? uq.p : nullptr, s2, o2, N, G, bits, want.p);
+  std::memset(y.p, 0xFF, n * 4);
+  std::memset(m.p, 0xFF, words * 4);
+  rc = exact_bn_relu_dropout_minmax_pack_f32(x.p, mean.p, mult.p, shift.p, p, supplied ? ua.p : nullptr, s1, o1,
+                                             supplied ? uq.p : nullptr, s2, o2, N, G, bits, y.p, m.p, packed.p, sc2.p,
+                                             mn2.p, sbf.p, mbf.p, nullptr);
+  bad = 0;
+  for (int64_t i = 0; i < words; ++i) bad += m[i] != (m1[i] & m2[i]);
+  CHECK(rc == 0 && std::memcmp(y.p, y2.p, n * 4) == 0 && bad == 0, "bn fused y/mask differ N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  CHECK(std::memcmp(packed.p, want.p, nb) == 0, "bn fused packed differs N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+  CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "bn fused scale/min differ N=%ld G=%ld", (long)N, (long)G);
 }
 
 // fp16 entry points against straight loops written here with _Float16 (the

@@ -224,8 +224,9 @@ def relu_dropout_fwd(x, prob, noise=None, seed=0, offset=0, guard=8):
 
 
 def relu_dropout_minmax_pack(x, prob, bits, act_noise=None, noise=None, act_seed=0, act_offset=0, seed=0, offset=0,
-                             guard=64, expect_rc=0):
-    """-> (y, mask words, packed, scale f32, min f32, scale bf16 bits, min bf16 bits)."""
+                             guard=64, expect_rc=0, norm=None):
+    """-> (y, mask words, packed, scale f32, min f32, scale bf16 bits, min bf16 bits).
+    norm = (mean, mult, shift) selects the entry point with batch norm ahead of the ReLU."""
     x = f32(x)
     N, G = x.shape
     n = N * G
@@ -238,9 +239,15 @@ def relu_dropout_minmax_pack(x, prob, bits, act_noise=None, noise=None, act_seed
     sbf, mbf = np.zeros(N, np.uint16), np.zeros(N, np.uint16)
     act_noise = None if act_noise is None else f32(act_noise)
     noise = None if noise is None else f32(noise)
-    rc = emu().exact_relu_dropout_minmax_pack_f32(p(x), prob, p(act_noise), act_seed, act_offset, p(noise), seed,
-                                                  offset, N, G, bits, p(y), p(mask), p(packed), p(s32), p(m32), p(sbf),
-                                                  p(mbf), None)
+    if norm is None:
+        rc = emu().exact_relu_dropout_minmax_pack_f32(p(x), prob, p(act_noise), act_seed, act_offset, p(noise), seed,
+                                                      offset, N, G, bits, p(y), p(mask), p(packed), p(s32), p(m32),
+                                                      p(sbf), p(mbf), None)
+    else:
+        mean, mult, shift = (None if v is None else f32(v) for v in norm)
+        rc = emu().exact_bn_relu_dropout_minmax_pack_f32(p(x), p(mean), p(mult), p(shift), prob, p(act_noise), act_seed,
+                                                         act_offset, p(noise), seed, offset, N, G, bits, p(y), p(mask),
+                                                         p(packed), p(s32), p(m32), p(sbf), p(mbf), None)
     assert rc == expect_rc, rc
     if rc != 0:
         return None

@@ -199,6 +199,42 @@ def test_relu_dropout_pack_kernel_equals_the_chain(N, G, bits, supplied):
         assert g_.tobytes() == w_.tobytes(), name
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("N,G", [(1, 8), (37, 40), (64, 256), (203, 256), (33, 1024), (129, 104)])
+@pytest.mark.parametrize("supplied", [True, False])
+def test_bn_relu_dropout_pack_kernel_equals_the_chain_on_the_normalised_input(N, G, bits, supplied):
+    rng = np.random.default_rng(N * 999 + G + bits)
+    x = (rng.standard_normal((N, G)) * 3 + 1).astype(F32)
+    mean = rng.standard_normal(G).astype(F32)
+    mult = (rng.random(G, dtype=F32) + F32(0.5)) * np.where(rng.random(G) < 0.2, F32(-1), F32(1)).astype(F32)
+    shift = rng.standard_normal(G).astype(F32)
+    if supplied:
+        act_noise, noise = rng.random((N, G), dtype=F32), rng.random((N, G), dtype=F32)
+    else:
+        act_noise = o.philox_noise_flat(21, 8, N * G).reshape(N, G)
+        noise = o.philox_noise_rows(22, 12, N, G)
+    got = e.relu_dropout_minmax_pack(x, 0.25, bits, act_noise if supplied else None, noise if supplied else None,
+                                     21, 8, 22, 12, norm=(mean, mult, shift))
+    normalised = ((x - mean[None, :]) * mult[None, :] + shift[None, :]).astype(F32)   # three fp32 roundings
+    want = _chain(normalised, 0.25, bits, act_noise, noise)
+    for name, g_, w_ in zip(("y", "mask", "packed", "scale", "min", "scale_bf16", "min_bf16"), got, want):
+        assert np.ascontiguousarray(g_).tobytes() == np.ascontiguousarray(w_).tobytes(), name
+    # the identity normalisation is the plain kernel
+    plain = e.relu_dropout_minmax_pack(x, 0.25, bits, act_noise if supplied else None, noise if supplied else None,
+                                       21, 8, 22, 12)
+    ident = e.relu_dropout_minmax_pack(x, 0.25, bits, act_noise if supplied else None, noise if supplied else None,
+                                       21, 8, 22, 12, norm=(np.zeros(G, F32), np.ones(G, F32), np.zeros(G, F32)))
+    for a_, b_ in zip(plain, ident):
+        assert np.ascontiguousarray(a_).tobytes() == np.ascontiguousarray(b_).tobytes()
+
+
+def test_bn_relu_dropout_pack_kernel_rejects_missing_vectors():
+    x = np.zeros((4, 16), F32)
+    v = np.zeros(16, F32)
+    assert e.relu_dropout_minmax_pack(x, 0.5, 2, norm=(v, None, v), expect_rc=-1) is None
+    assert e.relu_dropout_minmax_pack(np.zeros((4, 12), F32), 0.5, 2, norm=(v, v, v), expect_rc=-3) is None
+
+
 def test_relu_dropout_pack_kernel_rejects_what_it_cannot_do():
     x = np.zeros((4, 12), F32)
     assert e.relu_dropout_minmax_pack(x, 0.5, 2, expect_rc=-3) is None          # G % 8 != 0
@@ -209,12 +245,13 @@ def test_relu_dropout_pack_kernel_rejects_what_it_cannot_do():
 
 
 # ------------------------------------------------------------ fused epilogue (layers, both back ends)
-def _train_steps(backend, fuse, noise_seed, philox_seed, kept_frac=1.0, bits=2, steps=3, hidden=64):
+def _train_steps(backend, fuse, noise_seed, philox_seed, kept_frac=1.0, bits=2, steps=3, hidden=64, fold_bn=False):
     """A few SGD steps of a 3-layer GCN; -> (losses, final weights)."""
     from exact_amd.models import GCN
     from exact_amd.sparse import gcn_norm
     from gpu_util import SeededNoise
     config.fuse_epilogue = fuse
+    config.fold_batch_norm = fold_bn
     config.kept_frac = kept_frac
     config.activation_compression_bits = [bits]
     if noise_seed is None:
