@@ -71,12 +71,16 @@ def test_folded_batch_norm_matches_the_separate_layers(backend, N, G, affine, mo
     for (ys, dxs, dws, dbs), (yf, dxf, dwf, dbf) in zip(sep, fus):
         # elements within rounding of zero may land on either side of the ReLU: equal to 1e-5 all the same
         assert torch.allclose(ys, yf, rtol=1e-5, atol=2e-5)
-        flipped = ((ys != 0) != (yf != 0)).float().mean().item()
-        assert flipped < 1e-3
-        assert torch.allclose(dxs, dxf, rtol=1e-3, atol=1e-3 * dxs.abs().max().item())
+        flipped = (ys != 0) != (yf != 0)
+        assert flipped.float().mean().item() < 1e-3
+        # a flipped element changes the gradients of its whole column (batch norm's backward sums over the
+        # column); columns are independent, so the others must agree
+        same = ~flipped.any(0)
+        assert same.float().mean().item() > 0.9
+        assert torch.allclose(dxs[:, same], dxf[:, same], rtol=1e-3, atol=1e-3 * dxs.abs().max().item())
         if affine:
-            assert torch.allclose(dws, dwf, rtol=1e-3, atol=1e-3 * dws.abs().max().item())
-            assert torch.allclose(dbs, dbf, rtol=1e-3, atol=1e-3 * dbs.abs().max().item())
+            assert torch.allclose(dws[same], dwf[same], rtol=1e-3, atol=1e-3 * dws.abs().max().item())
+            assert torch.allclose(dbs[same], dbf[same], rtol=1e-3, atol=1e-3 * dbs.abs().max().item())
     if track:
         assert torch.allclose(sep_stats[0], fus_stats[0], rtol=1e-5, atol=1e-6)
         assert torch.allclose(sep_stats[1], fus_stats[1], rtol=1e-5, atol=1e-6)
