@@ -45,6 +45,8 @@ SIGNATURES = {
                                                     _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
     "exact_bn_relu_dropout_minmax_pack_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_f32, _c_ptr, _c_u64, _c_u64, _c_ptr, _c_u64, _c_u64,
                                                        _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
+    "exact_rp_minmax_pack_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                                          _c_ptr, _c_ptr, _c_ptr]),
     "exact_minmax_pack_f16": (_c_int, [_c_ptr, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
     "exact_unpack_f16": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_relu_fwd_f16": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr]),

@@ -152,6 +152,11 @@ def kernel_extras(x, log):
         q = ops.quantize_activation(xr_small, None)
         t = event_time(lambda: ops.quantize_activation(ops.input2rp(x, k)[0], None))
         out["rp_compress_int2"] = {"us": t * 1e6}
+        # the same in one launch: the [N, k] product is quantised in the accumulators
+        fused_bytes = 4 * N * G + 4 * G * k + (2 * N * k) // 8 + 4 * N
+        t_one = event_time(lambda: ops.project_and_quantize(x, None))
+        out["rp_pack_int2"] = {"us": t_one * 1e6, "GB/s": fused_bytes / t_one / 1e9, "algo_bytes": fused_bytes,
+                               "replaces_us": t * 1e6}
         t = event_time(lambda: ops.rp2input(ops.dequantize_activation(q, xr_small.shape), x.shape, R))
         out["rp_decompress_int2"] = {"us": t * 1e6}
         for name, v in out.items():
@@ -343,7 +348,7 @@ def _profile_target(argv=None):
     `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
 
         python -m exact_amd.benchmarks pack --bits 2 --reps 100
-        python -m exact_amd.benchmarks {unpack,relu,dropout,rp_fwd,rp_bwd,spmm,copy} ...
+        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy} ...
         python -m exact_amd.benchmarks epoch --config cfg3_gcn_int2 --epochs 5
 
     `copy` is a plain device-to-device copy of the same [rows, cols] fp32 tensor
@@ -359,7 +364,8 @@ def _profile_target(argv=None):
     if argv and argv[0] == "epoch":
         return _epoch_main(argv[1:])
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
-    ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "rp_fwd", "rp_bwd", "spmm", "copy"])
+    ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "relu_dropout_pack", "bn_relu_dropout_pack", "rp_fwd", "rp_bwd",
+                                      "rp_pack", "spmm", "copy"])
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--rows", type=int, default=169343)
     ap.add_argument("--cols", type=int, default=256)
@@ -383,6 +389,8 @@ def _profile_target(argv=None):
     k = int(0.125 * G + 0.999)
     R = torch.randn(G, k, generator=gen, device=dev) / k ** 0.5
     xr = torch.empty((N, k), device=dev)
+    packed_k = torch.empty(int(L.exact_packed_nbytes(N, k, b)), dtype=torch.int8, device=dev)
+    ones = torch.ones(G, device=dev)
     if args.kernel == "spmm":
         adj = gcn_norm(powerlaw_graph(N, int(N * 6.85), seed=1, device=dev)).to_int32_()
         rowptr, col, value = adj.csr()
@@ -395,6 +403,15 @@ def _profile_target(argv=None):
         "relu": lambda i: L.exact_relu_fwd_f32(x.data_ptr(), N * G, out.data_ptr(), mask.data_ptr(), sp),
         "dropout": lambda i: L.exact_dropout_fwd_f32(x.data_ptr(), None, 1, i, 0.5, N * G, out.data_ptr(),
                                                      mask.data_ptr(), sp),
+        "relu_dropout_pack": lambda i: L.exact_relu_dropout_minmax_pack_f32(
+            x.data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G, b, out.data_ptr(), mask.data_ptr(),
+            packed.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp),
+        "bn_relu_dropout_pack": lambda i: L.exact_bn_relu_dropout_minmax_pack_f32(
+            x.data_ptr(), ones.data_ptr(), ones.data_ptr(), ones.data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G,
+            b, out.data_ptr(), mask.data_ptr(), packed.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp),
+        "rp_pack": lambda i: L.exact_rp_minmax_pack_f32(x.data_ptr(), R.data_ptr(), None, 1, i, N, G, k, b,
+                                                        packed_k.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(),
+                                                        sp),
         "rp_fwd": lambda i: L.exact_rp_fwd_f32(x.data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp),
         "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, out.data_ptr(), sp),
         "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, x, "sum"),
@@ -402,7 +419,9 @@ def _profile_target(argv=None):
     }
     fn = fns[args.kernel]
     for i in range(args.reps):
-        fn(i + 2)
+        rc = fn(i + 2)
+        if isinstance(rc, int) and rc != 0:
+            raise RuntimeError(f"{args.kernel}: entry point returned {rc}")
     _sync()
     print(f"{args.kernel}: {args.reps} launches on [{N}, {G}] done")
 

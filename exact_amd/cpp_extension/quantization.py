@@ -166,6 +166,35 @@ def minmax_pack(data, bits, want_fp32=False):
     return packed, scale_bf, min_bf
 
 
+RP_PACK_MAX_COLUMNS = 128
+
+
+def rp_minmax_pack(data, rand_matrix, bits):
+    """minmax_pack of the projection data[N, D] . rand_matrix[D, k] in one launch:
+    the [N, k] product is quantised in the registers that accumulate it
+    (input2rp then quantize_activation, ops.py:141-149; k <= 128)
+    -> (packed int8, scale bf16, min bf16)."""
+    check_device_tensor(data, "data", 2)
+    check_device_tensor(rand_matrix, "rand_matrix", 2)
+    _check_bits(bits)
+    N, D = data.shape
+    if rand_matrix.shape[0] != D:
+        raise RuntimeError("rand_matrix does not match the input")
+    k = rand_matrix.shape[1]
+    if not 0 < k <= RP_PACK_MAX_COLUMNS:
+        raise RuntimeError(f"rp_minmax_pack takes 1 to {RP_PACK_MAX_COLUMNS} projected columns")
+    dev = data.device
+    packed = torch.empty(packed_nbytes(N, k, bits), dtype=torch.int8, device=dev)
+    scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
+    noise, seed, offset = _noise_for((N, k), dev)
+    rc = _lib.lib().exact_rp_minmax_pack_f32(ptr(data), ptr(rand_matrix), ptr(noise), seed, offset, N, D, k, bits,
+                                             ptr(packed), None, None, ptr(scale_bf), ptr(min_bf),
+                                             _checks.stream_ptr(data))
+    _lib.check(rc, "rp_minmax_pack")
+    return packed, scale_bf, min_bf
+
+
 def unpack_bf16param(data, bits, scale_bf16, min_bf16, N, group_size):
     """unpack_single_precision with the bf16 -> fp32 widening of
     dequantize_activation (ops.py:92-96) folded into the kernel."""

@@ -40,6 +40,51 @@ __device__ __forceinline__ void load_k_slice(const float* __restrict__ p, int kk
   }
 }
 
+// The main loop of rp_fwd_kernel for the kernel that goes on to quantise the
+// product: acc = X[row0 .. row0 + 31, :] . R for the calling wavefront; Rl is
+// the workgroup's LDS staging area [kFwdDChunk][NT * 32].  Every wavefront of
+// the workgroup must call it (it contains workgroup barriers).
+template <int VEC, int NT>
+__device__ __forceinline__ void rp_fwd_accumulate(const float* __restrict__ X, const float* __restrict__ R,
+                                                  int64_t N, int D, int k, float* Rl, floatx16 (&acc)[NT]) {
+  constexpr int KP = NT * kTile;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kTile;
+  const int64_t my_row = (row0 + l32 < N) ? row0 + l32 : N - 1;
+  const float* xrow = X + my_row * D;
+
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+
+  for (int dc = 0; dc < D; dc += kFwdDChunk) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < kFwdDChunk * KP; idx += kBlock) {
+      const int rr = idx / KP, cc = idx - rr * KP;
+      Rl[idx] = (dc + rr < D && cc < k) ? R[static_cast<int64_t>(dc + rr) * k + cc] : 0.f;
+    }
+    __syncthreads();
+    const int dlim = (D - dc < kFwdDChunk) ? D - dc : kFwdDChunk;
+    for (int kb = 0; kb < dlim; kb += 2 * VEC) {
+      const int ks = kb + VEC * half;  // this lane's k-slice inside the chunk
+      float a[VEC];
+      load_k_slice<VEC>(xrow, dc + ks, D, a);
+#pragma unroll
+      for (int t = 0; t < VEC; ++t) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const float b = Rl[(ks + t) * KP + nt * kTile + l32];
+          acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b, acc[nt], 0, 0, 0);
+        }
+      }
+    }
+  }
+}
+
 // out[N, k] = X[N, D] . R[D, k];  NT * 32 >= k columns per wavefront.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kBlock) void rp_fwd_kernel(const float* __restrict__ X,
@@ -95,6 +140,146 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_kernel(const float* __restrict_
   }
 }
 
+// ---------------------------------------------------------------------------
+// Projection and quantisation in one launch: the [N, k] product stays in the
+// accumulators, where its per-row min / range, the stochastic rounding and the
+// bit-packing of quantize_activation (ops.py:69-83; kernel
+// quantization_cuda_kernel.cu:63-94) are applied to it -- what
+// exact_rp_fwd_f32 followed by exact_minmax_pack_f32 computes, bit for bit,
+// without the [N, k] tensor ever reaching memory.
+//
+// In the accumulator layout a lane holds, per 32-column tile, one column of 16
+// rows: rows 4h .. 4h + 3 of each block of 8 (h = lane / 32).  So the row
+// statistics are butterflies over the 32 lanes of a half-wave; the 2, 4 or 8
+// rows that share a packed byte sit in one lane (8 rows: in the two lanes
+// l and l + 32); and lane l % 32 writes the byte of column l: 32 consecutive
+// bytes per row group.
+//
+// Noise: element (n, d) takes 16-bit half d % 8 of Philox block (d / 8, n), the
+// row stream of the pack kernel.  The 8 lanes that share d / 8 compute the
+// blocks of four rows at a time between them and hand the words round.
+struct RpPackArgs {
+  const float* X;
+  const float* R;
+  const float* noise;  // nullable: [N, k] uniforms
+  uint32_t seed_lo, seed_hi, off_lo, off_hi;
+  int64_t N;
+  int D, k, bits;
+  uint8_t* packed;
+  int64_t pad_index;
+  float* scale_f32;
+  float* min_f32;
+  uint16_t* scale_bf16;
+  uint16_t* min_bf16;
+};
+
+template <int VEC, int NT, bool NOISE_IN>
+__global__ __launch_bounds__(kBlock) void rp_fwd_pack_kernel(const RpPackArgs a) {
+  HIP_DYNAMIC_SHARED(float, Rl)  // [kFwdDChunk][NT * 32]
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kTile;
+  const int k = a.k;
+  const float B = static_cast<float>((1 << a.bits) - 1);
+
+  floatx16 acc[NT];
+  rp_fwd_accumulate<VEC, NT>(a.X, a.R, a.N, a.D, k, Rl, acc);
+
+  // The 16 accumulator rows are handled as four blocks of four consecutive rows
+  // (rows 8 * vg + 4 * half + 0 .. 3), the unit in which they share packed bytes;
+  // one block at a time keeps the epilogue within the registers of the main loop.
+  const int i8 = l32 & 7;            // position in the 8-lane group = element of a Philox block
+  const int group_first = lane & ~7;
+#pragma unroll
+  for (int vg = 0; vg < 4; ++vg) {
+    const int64_t rbase = row0 + 8 * vg + 4 * half;  // first of the four rows
+    // ---- row statistics: min / max over the k columns, then scale -----------
+    float mnv[4], sc[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float lo = __builtin_inff(), hi = -__builtin_inff();
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        if (nt * kTile + l32 < k) {
+          lo = fminf(lo, acc[nt][4 * vg + r]);
+          hi = fmaxf(hi, acc[nt][4 * vg + r]);
+        }
+      }
+      group_minmax(lo, hi, kTile);
+      mnv[r] = lo;
+      const float recip = 1.0f / (hi - lo);  // ops.py:39: reciprocal, then * B -- two roundings
+      sc[r] = recip * B;
+      if (l32 == 0 && rbase + r < a.N) {
+        if (a.scale_f32) a.scale_f32[rbase + r] = sc[r];
+        if (a.min_f32) a.min_f32[rbase + r] = lo;
+        if (a.scale_bf16) a.scale_bf16[rbase + r] = f32_to_bf16_rne(sc[r]);
+        if (a.min_bf16) a.min_bf16[rbase + r] = f32_to_bf16_rne(lo);
+      }
+    }
+
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int cj = nt * kTile + l32;
+      const bool col_ok = cj < k;
+      // ---- noise -------------------------------------------------------------
+      float u[4];
+      if constexpr (NOISE_IN) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) u[r] = (col_ok && rbase + r < a.N) ? a.noise[(rbase + r) * k + cj] : 0.f;
+      } else {
+        // lane i8 of an 8-lane group computes the block of row i8 % 4 (twice over
+        // the group), then every lane fetches the word holding its element
+        const Philox4 mine = philox4x32_10(static_cast<uint32_t>(cj >> 3), static_cast<uint32_t>(rbase + (i8 & 3)),
+                                           a.off_lo, a.off_hi, a.seed_lo, a.seed_hi);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int src = group_first | r;
+          const uint32_t w0 = __shfl(mine.x, src), w1 = __shfl(mine.y, src), w2 = __shfl(mine.z, src),
+                         w3 = __shfl(mine.w, src);
+          const uint32_t lo_pair = (i8 & 2) ? w1 : w0, hi_pair = (i8 & 2) ? w3 : w2;
+          const uint32_t word = (i8 & 4) ? hi_pair : lo_pair;
+          u[r] = u16_to_uniform((i8 & 1) ? (word >> 16) : (word & 0xFFFFu));
+        }
+      }
+      // ---- quantise (quantization_cuda_kernel.cu:89, one rounding per operation) --
+      uint32_t q[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float tq = acc[nt][4 * vg + r] - mnv[r];
+        tq = tq * sc[r];
+        tq = tq + u[r];
+        tq = tq - 0.5f;
+        tq = fmaxf(tq, 0.f);
+        const uint32_t qi = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
+        q[r] = (col_ok && rbase + r < a.N) ? (qi & 0xFFu) : 0u;
+      }
+      // ---- pack: byte (n / wpt) * k + d holds rows n .. n + wpt - 1 of column d ----
+      if (a.bits == 8) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (col_ok && rbase + r < a.N) a.packed[(rbase + r) * k + cj] = static_cast<uint8_t>(q[r]);
+      } else if (a.bits == 4) {
+#pragma unroll
+        for (int r = 0; r < 4; r += 2)
+          if (col_ok && rbase + r < a.N) a.packed[((rbase + r) >> 1) * k + cj] = static_cast<uint8_t>(q[r] | (q[r + 1] << 4));
+      } else if (a.bits == 2) {
+        if (col_ok && rbase < a.N)
+          a.packed[(rbase >> 2) * k + cj] = static_cast<uint8_t>(q[0] | (q[1] << 2) | (q[2] << 4) | (q[3] << 6));
+      } else {
+        const uint32_t nib = q[0] | (q[1] << 1) | (q[2] << 2) | (q[3] << 3);  // rows 4 * half .. 4 * half + 3 of the eight
+        const uint32_t other = __shfl_xor(nib, 32);
+        const uint32_t byte = half ? (other | (nib << 4)) : (nib | (other << 4));
+        const int64_t first = row0 + 8 * vg;
+        // the two half-waves hold the same byte: they take turns storing
+        if (col_ok && first < a.N && (vg & 1) == half) a.packed[(first >> 3) * k + cj] = static_cast<uint8_t>(byte);
+      }
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) a.packed[a.pad_index] = 0;
+}
+
 // out[N, D] = Xr[N, k] . R[D, k]^T;  grid.y tiles D in slabs of NT * 32 columns.
 template <int VEC, int NT>
 __global__ __launch_bounds__(kBlock) void rp_bwd_kernel(const float* __restrict__ Xr,
@@ -148,6 +333,8 @@ __global__ __launch_bounds__(kBlock) void rp_bwd_kernel(const float* __restrict_
   }
 }
 
+__global__ void rp_zero_byte_kernel(uint8_t* p) { *p = 0; }
+
 static bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static bool al8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
 
@@ -161,6 +348,21 @@ static int rp_fwd_launch(const float* X, const float* R, int64_t N, int D, int k
     case 2: hipLaunchKernelGGL((rp_fwd_kernel<VEC, 2>), grid, dim3(kBlock), lds, s, X, R, N, D, k, out); break;
     case 3: hipLaunchKernelGGL((rp_fwd_kernel<VEC, 3>), grid, dim3(kBlock), lds, s, X, R, N, D, k, out); break;
     case 4: hipLaunchKernelGGL((rp_fwd_kernel<VEC, 4>), grid, dim3(kBlock), lds, s, X, R, N, D, k, out); break;
+    default: return EXACT_E_SHAPE;
+  }
+  return launch_status();
+}
+
+template <int VEC, bool NOISE_IN>
+static int rp_fwd_pack_launch(const RpPackArgs& a, hipStream_t s) {
+  const int nt = (a.k + kTile - 1) / kTile;
+  const dim3 grid(static_cast<unsigned>((a.N + 127) / 128));
+  const size_t lds = static_cast<size_t>(kFwdDChunk) * nt * kTile * sizeof(float);
+  switch (nt) {
+    case 1: hipLaunchKernelGGL((rp_fwd_pack_kernel<VEC, 1, NOISE_IN>), grid, dim3(kBlock), lds, s, a); break;
+    case 2: hipLaunchKernelGGL((rp_fwd_pack_kernel<VEC, 2, NOISE_IN>), grid, dim3(kBlock), lds, s, a); break;
+    case 3: hipLaunchKernelGGL((rp_fwd_pack_kernel<VEC, 3, NOISE_IN>), grid, dim3(kBlock), lds, s, a); break;
+    case 4: hipLaunchKernelGGL((rp_fwd_pack_kernel<VEC, 4, NOISE_IN>), grid, dim3(kBlock), lds, s, a); break;
     default: return EXACT_E_SHAPE;
   }
   return launch_status();
@@ -193,6 +395,41 @@ int exact_rp_fwd_f32(const float* X, const float* R, int64_t N, int64_t D, int64
   if (D % 4 == 0 && al16(X)) return rp_fwd_launch<4>(X, R, N, static_cast<int>(D), static_cast<int>(k), out, s);
   if (D % 2 == 0 && al8(X)) return rp_fwd_launch<2>(X, R, N, static_cast<int>(D), static_cast<int>(k), out, s);
   return rp_fwd_launch<1>(X, R, N, static_cast<int>(D), static_cast<int>(k), out, s);
+}
+
+int exact_rp_minmax_pack_f32(const float* X, const float* R, const float* noise, uint64_t seed, uint64_t offset,
+                             int64_t N, int64_t D, int64_t k, int bits, uint8_t* packed, float* scale_f32,
+                             float* min_f32, uint16_t* scale_bf16, uint16_t* min_bf16, void* stream) {
+  if (bits != 1 && bits != 2 && bits != 4 && bits != 8) return EXACT_E_BITS;
+  if (N < 0 || D <= 0 || k <= 0 || D > (1 << 20) || k > 128 || N > (int64_t{1} << 31) - 64) return EXACT_E_SHAPE;
+  if (!packed) return EXACT_E_NULL;
+  RpPackArgs a{};
+  a.pad_index = exact_packed_nbytes(N, k, bits) - 1;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (N == 0) {
+    hipLaunchKernelGGL(rp_zero_byte_kernel, dim3(1), dim3(1), 0, s, packed + a.pad_index);
+    return launch_status();
+  }
+  if (!X || !R) return EXACT_E_NULL;
+  a.X = X;
+  a.R = R;
+  a.noise = noise;
+  a.seed_lo = static_cast<uint32_t>(seed);
+  a.seed_hi = static_cast<uint32_t>(seed >> 32);
+  a.off_lo = static_cast<uint32_t>(offset);
+  a.off_hi = static_cast<uint32_t>(offset >> 32);
+  a.N = N;
+  a.D = static_cast<int>(D);
+  a.k = static_cast<int>(k);
+  a.bits = bits;
+  a.packed = packed;
+  a.scale_f32 = scale_f32;
+  a.min_f32 = min_f32;
+  a.scale_bf16 = scale_bf16;
+  a.min_bf16 = min_bf16;
+  if (D % 4 == 0 && al16(X)) return noise ? rp_fwd_pack_launch<4, true>(a, s) : rp_fwd_pack_launch<4, false>(a, s);
+  if (D % 2 == 0 && al8(X)) return noise ? rp_fwd_pack_launch<2, true>(a, s) : rp_fwd_pack_launch<2, false>(a, s);
+  return noise ? rp_fwd_pack_launch<1, true>(a, s) : rp_fwd_pack_launch<1, false>(a, s);
 }
 
 int exact_rp_bwd_f32(const float* Xr, const float* R, int64_t N, int64_t D, int64_t k, float* out,

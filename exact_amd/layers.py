@@ -15,7 +15,7 @@ from torch.nn import Parameter
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCN2Conv, GCNConv, GENConv, GraphConv, SAGEConv, glorot
-from .ops import (bn_relu_dropout, consumer_bits, input2rp, kept_columns, qbatch_norm, qelu, qlinear,
+from .ops import (bn_relu_dropout, consumer_bits, project_and_quantize, qbatch_norm, qelu, qlinear,
                   quantize_activation, relu_dropout, take_compressed)
 from .qsheme import QScheme
 from .spmm import QMatmul, qmatmul
@@ -135,8 +135,8 @@ class QSAGEConv(SAGEConv):
         if handed_over is not None:
             return handed_over, None
         if config.kept_frac < 1.0:
-            reduced, randmat = input2rp(x, kept_columns(x.shape[1]))
-            return quantize_activation(reduced, self.scheme), randmat
+            quantized, randmat, _ = project_and_quantize(x, self.scheme)
+            return quantized, randmat
         return quantize_activation(x, self.scheme), None
 
     def forward(self, x, edge_index, size=None):

@@ -134,6 +134,9 @@ def _projection_matrix(D, k, device, dtype):
     return (2.0 * signs - 1) / k ** 0.5
 
 
+RP_KERNEL_MAX_COLUMNS = 128      # k of exact_rp_fwd_f32 / exact_rp_bwd_f32 / exact_rp_minmax_pack_f32
+
+
 def kept_columns(width):
     """k of the projection D -> k (reference ops.py:143)."""
     return int(config.kept_frac * width + 0.999)
@@ -146,8 +149,9 @@ def input2rp(input, kept_acts):  # noqa: A002
     check_device_tensor(input, "input", 2, FLOAT_OR_HALF)
     N, D = input.shape
     rand_matrix = _projection_matrix(D, kept_acts, input.device, input.dtype).contiguous()
-    if input.dtype != torch.float32:
-        # fp16 activations (autocast): a plain library GEMM, as torch.matmul is in the reference
+    if input.dtype != torch.float32 or kept_acts > RP_KERNEL_MAX_COLUMNS:
+        # fp16 activations (autocast), or more projected columns than the kernel's
+        # accumulators hold: a plain library GEMM, as torch.matmul is in the reference
         return torch.matmul(input, rand_matrix), rand_matrix
     reduced = torch.empty((N, kept_acts), dtype=input.dtype, device=input.device)
     rc = _lib.lib().exact_rp_fwd_f32(ptr(input), ptr(rand_matrix), N, D, kept_acts, ptr(reduced),
@@ -162,7 +166,7 @@ def rp2input(dim_reduced_input, input_shape, rand_matrix):
     assert dim_reduced_input.dim() == 2
     check_device_tensor(dim_reduced_input, "dim_reduced_input", 2, FLOAT_OR_HALF)
     check_device_tensor(rand_matrix, "rand_matrix", 2, (dim_reduced_input.dtype,))
-    if dim_reduced_input.dtype != torch.float32:
+    if dim_reduced_input.dtype != torch.float32 or dim_reduced_input.shape[1] > RP_KERNEL_MAX_COLUMNS:
         return torch.matmul(dim_reduced_input, rand_matrix.t()).view(input_shape)
     N, k = dim_reduced_input.shape
     D = rand_matrix.shape[0]
@@ -173,6 +177,30 @@ def rp2input(dim_reduced_input, input_shape, rand_matrix):
                                      _checks.stream_ptr(dim_reduced_input))
     _lib.check(rc, "rp2input")
     return full.view(input_shape)
+
+
+def project_and_quantize(input, scheme):  # noqa: A002
+    """input2rp followed by quantize_activation of the result (reference
+    ops.py:141-149, layers.py:153-159) -> (quantized, rand_matrix, reduced shape).
+    One launch that never writes the [N, k] product where the kernel applies
+    (fp32, k <= 128, compression on), bit-identical to the two calls, which
+    run otherwise."""
+    k = kept_columns(input.shape[1])
+    fused = (config.fuse_epilogue and config.compress_activation and not config.simulate
+             and input.dim() == 2 and input.dtype == torch.float32 and not torch.is_autocast_enabled()
+             and 0 < k <= ext_quantization.RP_PACK_MAX_COLUMNS)
+    if not fused:
+        reduced, rand_matrix = input2rp(input, k)
+        return quantize_activation(reduced, scheme), rand_matrix, reduced.shape
+    check_device_tensor(input, "input", 2)
+    rand_matrix = _projection_matrix(input.shape[1], k, input.device, input.dtype).contiguous()
+    if scheme:
+        scheme.note_use()
+    bits = config.activation_compression_bits[0]
+    packed, scale_bf16, min_bf16 = ext_quantization.rp_minmax_pack(input, rand_matrix, bits)
+    if config.swap:
+        packed = swap_to_cpu(packed)
+    return (packed, bits, scale_bf16, min_bf16), rand_matrix, torch.Size((input.shape[0], k))
 
 
 class CompressedActivation:
@@ -191,8 +219,8 @@ class CompressedActivation:
         """Project (when kept_frac < 1 and allowed) and quantise x
         (reference ops.py:141-149, 272-280, 326-334)."""
         if project and config.kept_frac < 1.0:
-            reduced, randmat = input2rp(x, kept_columns(x.shape[1]))
-            return cls(quantize_activation(reduced, scheme), randmat, x.shape, reduced.shape)
+            quantized, randmat, stored_shape = project_and_quantize(x, scheme)
+            return cls(quantized, randmat, x.shape, stored_shape)
         return cls(quantize_activation(x, scheme), None, x.shape, x.shape)
 
     @classmethod

@@ -261,6 +261,18 @@ int exact_rp_fwd_f32(const float *X, const float *R, int64_t N, int64_t D,
 int exact_rp_bwd_f32(const float *Xr, const float *R, int64_t N, int64_t D,
                      int64_t k, float *out, void *stream);
 
+/* Projection and quantisation in one launch: what exact_rp_fwd_f32 followed by
+ * exact_minmax_pack_f32 (on the [N, k] product, G = k) computes, bit for bit,
+ * without the [N, k] tensor reaching memory -- input2rp then
+ * quantize_activation as qlinear.forward and QSAGEConv.forward chain them
+ * (ops.py:141-149, layers.py:153-159).  k <= 128.  noise: NULL or [N, k]
+ * uniforms; seed / offset, packed, scale and min outputs as in
+ * exact_minmax_pack_f32 (packed holds exact_packed_nbytes(N, k, bits) bytes). */
+int exact_rp_minmax_pack_f32(const float *X, const float *R, const float *noise, uint64_t seed,
+                             uint64_t offset, int64_t N, int64_t D, int64_t k, int bits,
+                             uint8_t *packed, float *scale_f32, float *min_f32,
+                             uint16_t *scale_bf16, uint16_t *min_bf16, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -184,6 +184,26 @@ static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
   worst = 0, scale = 1e-30;
   for (int64_t i = 0; i < N * D; ++i) { scale = std::max(scale, (double)std::fabs(wback[i])); worst = std::max(worst, (double)std::fabs(back[i] - wback[i])); }
   CHECK(worst <= 2e-5 * scale, "rp bwd differs N=%ld D=%ld k=%ld: %g of %g", (long)N, (long)D, (long)k, worst, scale);
+  // projection + quantisation in one launch == the oracle's quantiser on the kernel's own product
+  std::uniform_real_distribution<float> ud(0.f, 1.f);
+  Buf<float> u(N * k), mn(N), mx(N), sc(N), mn2(N), sc2(N);
+  for (int64_t i = 0; i < N * k; ++i) { u[i] = ud(rng); if (u[i] >= 1.f) u[i] = 0.5f; }
+  oracle_row_minmax(xr.p, N, k, mn.p, mx.p);
+  for (int bits : {1, 2, 4, 8}) {
+    const bool supplied = bits == 2 || bits == 8;
+    const int64_t nb = exact_packed_nbytes(N, k, bits);
+    Buf<uint8_t> packed(nb), want(nb);
+    Buf<uint16_t> sbf(N), mbf(N);
+    oracle_scale(mn.p, mx.p, N, bits, sc.p);
+    std::memset(want.p, 0, nb);
+    oracle_pack(xr.p, mn.p, sc.p, supplied ? u.p : nullptr, 0x99ull, (7ull << 32) + 16, N, k, bits, want.p);
+    std::memset(packed.p, 0xEE, nb);
+    const int rc = exact_rp_minmax_pack_f32(X.p, R.p, supplied ? u.p : nullptr, 0x99ull, (7ull << 32) + 16, N, D, k, bits,
+                                            packed.p, sc2.p, mn2.p, sbf.p, mbf.p, nullptr);
+    CHECK(rc == 0 && std::memcmp(packed.p, want.p, nb) == 0, "rp+pack packed differs N=%ld D=%ld k=%ld bits=%d rc=%d",
+          (long)N, (long)D, (long)k, bits, rc);
+    CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "rp+pack scale/min differ N=%ld k=%ld", (long)N, (long)k);
+  }
 }
 
 // LeakyReLU mask, max / min aggregation and the edge-value gradient, against

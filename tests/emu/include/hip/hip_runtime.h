@@ -284,6 +284,16 @@ inline uint32_t shfl_xor_u32(uint32_t v, int m) {
   return static_cast<uint32_t>(w->slot[buf][src]);
 }
 
+// __shfl with the default width: every lane names the lane it reads (ds_bpermute)
+inline uint32_t shfl_u32(uint32_t v, int src) {
+  WaveState* w;
+  int lane;
+  const int buf = wave_collect(v, w, lane);
+  src &= kWaveSize - 1;
+  if (!((w->mask[buf] >> src) & 1)) return v;
+  return static_cast<uint32_t>(w->slot[buf][src]);
+}
+
 inline uint32_t readlane_u32(uint32_t v, int src) {
   WaveState* w;
   int lane;
@@ -441,6 +451,7 @@ static inline float __shfl_xor(float v, int m) {
 }
 static inline uint32_t __shfl_xor(uint32_t v, int m) { return hipemu::shfl_xor_u32(v, m); }
 static inline int __shfl_xor(int v, int m) { return static_cast<int>(hipemu::shfl_xor_u32(static_cast<uint32_t>(v), m)); }
+static inline uint32_t __shfl(uint32_t v, int src) { return hipemu::shfl_u32(v, src); }
 static inline uint64_t __ballot(bool p) { return hipemu::ballot(p); }
 #define __builtin_amdgcn_readlane(v, l) static_cast<int>(hipemu::readlane_u32(static_cast<uint32_t>(v), (l)))
 #define __builtin_amdgcn_readfirstlane(v) static_cast<int>(hipemu::readfirstlane_u32(static_cast<uint32_t>(v)))

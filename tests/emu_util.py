@@ -157,6 +157,25 @@ def rp_fwd(X, R, guard=16):
     return out[:N * k].reshape(N, k)
 
 
+def rp_minmax_pack(X, R, bits, noise=None, seed=0, offset=0, guard=64, expect_rc=0):
+    """-> (packed, scale f32, min f32, scale bf16 bits, min bf16 bits) of the projected X."""
+    X, R = f32(X), f32(R)
+    N, D = X.shape
+    k = R.shape[1]
+    nb = int(emu().exact_packed_nbytes(N, k, bits)) if bits in (1, 2, 4, 8) else 1
+    packed = np.full(nb + guard, 0xA5, np.uint8)
+    s32, m32 = np.full(N + 1, np.float32(-3.0), np.float32), np.full(N + 1, np.float32(-3.0), np.float32)
+    sbf, mbf = np.full(N + 1, 0x1234, np.uint16), np.full(N + 1, 0x1234, np.uint16)
+    noise = None if noise is None else f32(noise)
+    rc = emu().exact_rp_minmax_pack_f32(p(X), p(R), p(noise), seed, offset, N, D, k, bits, p(packed), p(s32), p(m32),
+                                        p(sbf), p(mbf), None)
+    assert rc == expect_rc, rc
+    if rc != 0:
+        return None
+    assert (packed[nb:] == 0xA5).all() and s32[N] == -3.0 and m32[N] == -3.0 and sbf[N] == 0x1234 and mbf[N] == 0x1234
+    return packed[:nb], s32[:N], m32[:N], sbf[:N], mbf[:N]
+
+
 def rp_bwd(Xr, R, guard=16):
     Xr, R = f32(Xr), f32(R)
     N, k = Xr.shape

@@ -129,3 +129,11 @@ def test_epoch_entry_point(cpu_harness, capsys):
     bm._profile_target(["epoch", "--config", "cfg3_gcn_int2", "--epochs", "1", "--warmup", "0", "--scale", "0.0005"])
     res = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert res["epochs_per_s"] > 0 and res["bits"] == 2
+
+
+@pytest.mark.parametrize("kernel", ["pack", "unpack", "relu", "dropout", "relu_dropout_pack", "bn_relu_dropout_pack",
+                                    "rp_fwd", "rp_bwd", "rp_pack", "copy"])
+def test_kernel_trace_targets_run(cpu_harness, capsys, kernel):
+    """`python -m exact_amd.benchmarks <kernel>`: every target launches its entry point with valid arguments."""
+    bm._profile_target([kernel, "--rows", "70", "--cols", "64", "--reps", "2"])
+    assert f"{kernel}: 2 launches on [70, 64] done" in capsys.readouterr().out

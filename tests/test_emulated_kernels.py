@@ -139,6 +139,42 @@ def test_rp(N, D, frac, dist):
     np.testing.assert_allclose(back, wb, rtol=1e-5, atol=1e-5 * np.abs(wb).max())
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("supplied", [True, False])
+@pytest.mark.parametrize("N,D,frac", [(1, 256, 0.125), (31, 256, 0.125), (200, 256, 0.125), (130, 602, 0.125),
+                                      (140, 100, 0.25), (129, 256, 0.25), (64, 128, 0.5), (77, 50, 0.3), (130, 7, 0.5),
+                                      (100, 256, 0.49), (261, 602, 0.2)])
+def test_projection_and_quantisation_in_one_launch_equal_the_two_launches(N, D, frac, bits, supplied):
+    """exact_rp_minmax_pack_f32 == exact_rp_fwd_f32 followed by the oracle's
+    quantize_activation of that product, bit for bit (packed bytes, fp32 and
+    bf16 scale / min), with supplied noise and with the internal Philox stream."""
+    k = o.kept_acts(frac, D)
+    rng = np.random.default_rng(N * 7 + D + bits)
+    R = o.gaussian_matrix(D, k, rng)
+    X = rng.standard_normal((N, D)).astype(F32)
+    if N > 4:
+        X[3] = 0.0                                  # a constant (all-zero) projected row: scale = inf
+    reduced = e.rp_fwd(X, R)
+    noise = rng.random((N, k), dtype=F32) if supplied else o.philox_noise_rows(91, 4 * bits, N, k)
+    want_packed, _, want_sbf, want_mbf, want_scale, want_mn = o.quantize_activation(reduced, bits, noise)
+    packed, s32, m32, sbf, mbf = e.rp_minmax_pack(X, R, bits, noise if supplied else None, 91, 4 * bits)
+    assert np.array_equal(m32.view(np.uint32), want_mn.view(np.uint32))
+    assert np.array_equal(s32.view(np.uint32), want_scale.view(np.uint32))
+    assert np.array_equal(sbf, want_sbf) and np.array_equal(mbf, want_mbf)
+    assert packed[-1] == 0 and np.array_equal(packed[:-1], want_packed[:packed.size - 1])
+    # and it is what the stand-alone pack entry point makes of the product
+    alone = e.minmax_pack(reduced, bits, noise if supplied else None, 91, 4 * bits)
+    assert np.array_equal(alone[0], packed)
+
+
+def test_projection_and_quantisation_argument_checks():
+    X, R = np.zeros((4, 16), F32), np.zeros((16, 4), F32)
+    assert e.rp_minmax_pack(X, R, 3, expect_rc=-2) is None
+    assert e.rp_minmax_pack(np.zeros((4, 300), F32), np.zeros((300, 129), F32), 2, expect_rc=-3) is None
+    got = e.rp_minmax_pack(np.zeros((0, 16), F32), R, 2)
+    assert got[0].size == 1 and got[0][0] == 0
+
+
 def test_pack_unpack_random_shapes():
     """Randomly drawn shapes (any N, any G up to a few thousand, every bit
     width, both noise modes): the fixed list above cannot enumerate every
