@@ -40,14 +40,25 @@ __device__ __forceinline__ void load_k_slice(const float* __restrict__ p, int kk
   }
 }
 
-// The main loop of rp_fwd_kernel for the kernel that goes on to quantise the
-// product: acc = X[row0 .. row0 + 31, :] . R for the calling wavefront; Rl is
-// the workgroup's LDS staging area [kFwdDChunk][NT * 32].  Every wavefront of
-// the workgroup must call it (it contains workgroup barriers).
+// The product of rp_fwd_kernel for the kernel that goes on to quantise it:
+// acc = X[row0 .. row0 + 31, :] . R for the calling wavefront, the MFMA steps in
+// the same order (so the same bits).  Rl is the workgroup's LDS staging area
+// [kFwdDChunk][NT * 32]; every wavefront of the workgroup must call this (it
+// contains workgroup barriers).
+//
+// Memory-level parallelism: a lane issues the loads of its whole share of a
+// 64-column chunk (eight 16-byte loads at VEC = 4: the 128-byte line of its
+// row and the next) before the first MFMA consumes them, and the threads that
+// stage R fetch eight elements each before the first LDS write -- one exposure
+// to memory latency per chunk instead of one per load.
 template <int VEC, int NT>
 __device__ __forceinline__ void rp_fwd_accumulate(const float* __restrict__ X, const float* __restrict__ R,
                                                   int64_t N, int D, int k, float* Rl, floatx16 (&acc)[NT]) {
   constexpr int KP = NT * kTile;
+  constexpr int kBatch = 8;
+  constexpr int kStagePerThread = kFwdDChunk * KP / kBlock;  // 8 * NT
+  constexpr int kSteps = kFwdDChunk / (2 * VEC);             // k-slices of a lane per chunk
+  static_assert(kStagePerThread % kBatch == 0 && kSteps % kBatch == 0, "batches divide the chunk");
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const int half = lane >> 5;
@@ -63,22 +74,40 @@ __device__ __forceinline__ void rp_fwd_accumulate(const float* __restrict__ X, c
 
   for (int dc = 0; dc < D; dc += kFwdDChunk) {
     __syncthreads();
-    for (int idx = threadIdx.x; idx < kFwdDChunk * KP; idx += kBlock) {
-      const int rr = idx / KP, cc = idx - rr * KP;
-      Rl[idx] = (dc + rr < D && cc < k) ? R[static_cast<int64_t>(dc + rr) * k + cc] : 0.f;
+    for (int b0 = 0; b0 < kStagePerThread; b0 += kBatch) {
+      float staged[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        const int idx = threadIdx.x + (b0 + i) * kBlock;
+        const int rr = idx / KP, cc = idx - rr * KP;
+        staged[i] = (dc + rr < D && cc < k) ? R[static_cast<int64_t>(dc + rr) * k + cc] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) Rl[threadIdx.x + (b0 + i) * kBlock] = staged[i];
     }
     __syncthreads();
     const int dlim = (D - dc < kFwdDChunk) ? D - dc : kFwdDChunk;
-    for (int kb = 0; kb < dlim; kb += 2 * VEC) {
-      const int ks = kb + VEC * half;  // this lane's k-slice inside the chunk
-      float a[VEC];
-      load_k_slice<VEC>(xrow, dc + ks, D, a);
+    for (int s0 = 0; s0 < kSteps; s0 += kBatch) {
+      if (s0 * 2 * VEC >= dlim) break;
+      float a[kBatch][VEC];
 #pragma unroll
-      for (int t = 0; t < VEC; ++t) {
+      for (int sb = 0; sb < kBatch; ++sb) {
+        const int ks = (s0 + sb) * 2 * VEC + VEC * half;  // this lane's k-slice inside the chunk
+        load_k_slice<VEC>(xrow, dc + ks, D, a[sb]);        // zeros past column D
+      }
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const float b = Rl[(ks + t) * KP + nt * kTile + l32];
-          acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b, acc[nt], 0, 0, 0);
+      for (int sb = 0; sb < kBatch; ++sb) {
+        const int kb = (s0 + sb) * 2 * VEC;
+        if (kb < dlim) {
+          const int ks = kb + VEC * half;
+#pragma unroll
+          for (int t = 0; t < VEC; ++t) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              const float b = Rl[(ks + t) * KP + nt * kTile + l32];
+              acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[sb][t], b, acc[nt], 0, 0, 0);
+            }
+          }
         }
       }
     }

@@ -57,6 +57,14 @@ def quant_case(rng):
         y1, m1 = o.relu_fwd(x.reshape(-1)); y2, m2 = o.dropout_fwd(y1, 0.3, an.reshape(-1))
         w = o.quantize_activation(y2.reshape(N, G), bits, noise)
         assert np.array_equal(got[0].view(np.uint32), y2.reshape(N, G).view(np.uint32)) and np.array_equal(got[1], m1 & m2) and np.array_equal(got[2], w[0]), ("fused", N, G, bits, supplied)
+        # with batch norm ahead of the ReLU
+        mean, mult, shift = (rng.standard_normal(G).astype(F32) for _ in range(3))
+        got = e.relu_dropout_minmax_pack(x, 0.3, bits, an if supplied else None, noise if supplied else None, seed ^ 5, off + 4, seed, off,
+                                         norm=(mean, mult, shift))
+        xn = ((x - mean[None, :]) * mult[None, :] + shift[None, :]).astype(F32)
+        y1, m1 = o.relu_fwd(xn.reshape(-1)); y2, m2 = o.dropout_fwd(y1, 0.3, an.reshape(-1))
+        w = o.quantize_activation(y2.reshape(N, G), bits, noise)
+        assert np.array_equal(got[0].view(np.uint32), y2.reshape(N, G).view(np.uint32)) and np.array_equal(got[1], m1 & m2) and np.array_equal(got[2], w[0]), ("bn fused", N, G, bits, supplied)
 
 def other_case(rng, n):
     """masks, max / min aggregation, edge-value gradient, projection, two-step pack."""
@@ -96,6 +104,13 @@ def other_case(rng, n):
         assert np.allclose(a, w, rtol=2e-5, atol=2e-5 * np.abs(w).max()), ("rp_fwd", N, D, kk)
         b = e.rp_bwd(w, R); wb = o.rp2input(w, R)
         assert np.allclose(b, wb, rtol=2e-5, atol=2e-5 * np.abs(wb).max()), ("rp_bwd", N, D, kk)
+        # projection + quantisation in one launch == the oracle's quantiser on the kernel's own product
+        bits = int(rng.choice([1, 2, 4, 8])); supplied = bool(rng.integers(0, 2))
+        seed, off = int(rng.integers(0, 2**63)), int(rng.integers(0, 2**40))
+        noise = rng.random((N, kk), dtype=F32) if supplied else o.philox_noise_rows(seed, off, N, kk)
+        got = e.rp_minmax_pack(X, R, bits, noise if supplied else None, seed, off)
+        wq = o.quantize_activation(a, bits, noise)
+        assert np.array_equal(got[0][:-1], wq[0][:got[0].size - 1]) and np.array_equal(got[3], wq[2]) and np.array_equal(got[4], wq[3]), ("rp_pack", N, D, kk, bits, supplied)
     else:           # two-step pack with given min / scale, row_minmax
         N, G = int(rng.integers(1, 300)), int(rng.integers(1, 2200)); bits = int(rng.choice([1, 2, 4, 8]))
         x = rng.standard_normal((N, G)).astype(F32); mn, mx = o.row_min_max(x); sc = o.compute_scale(mn, mx, bits)
