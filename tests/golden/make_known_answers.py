@@ -86,6 +86,18 @@ CASES = [
      "y": [[0, 4, 0, 0, 10, 12, 14, 16]], "mask": [0xF2], "packed": [0, 1, 0, 0, 2, 2, 3, 3, 0],
      "scale_bf16": [0x3E40], "min_bf16": [0x0000]},
 
+    # ---- batch norm -> ReLU -> dropout -> minmax_pack as one call (layers.py:340-369 ahead of the chain) ----
+    # per column (x - mean) * mult + shift, all exact in fp32:
+    #   row 0 -> [-1, 2, 3, -4, 5, 6, 7, 8], the case above; row 1 -> [0.5, 0, 1, 0, 0, 6, 16, 0], nothing dropped:
+    #   y = [1, 0, 2, 0, 0, 12, 32, 0], mask bits 8, 10, 13, 14; mn 0, mx 32: scale = fl(1/32) * 3 = 0.09375;
+    #   codes rne([.09375, 0, .1875, 0, 0, 1.125, 3, 0]) = [0, 0, 0, 0, 0, 1, 3, 0]; byte d = row 0 | row 1 << 2
+    {"op": "bn_relu_dropout_pack", "p": 0.5, "bits": 2,
+     "x": [[0.25, 2, 3, 4, 1, 10, 0, 0], [1, 0, -1, 2, 0, 10, 9, -8]],
+     "mean": [1, 0, -1, 2, 0, 10, 0, -8], "mult": [2, 1, 0.5, -2, 5, 1, 1, 1], "shift": [0.5, 0, 1, 0, 0, 6, 7, 0],
+     "act_noise": [[0.9, 0.9, 0.1, 0.9, 0.9, 0.9, 0.9, 0.9], [0.9] * 8], "noise": [[HALF] * 8] * 2,
+     "y": [[0, 4, 0, 0, 10, 12, 14, 16], [1, 0, 2, 0, 0, 12, 32, 0]], "mask": [0x65F2],
+     "packed": [0, 1, 0, 0, 2, 6, 15, 3, 0], "scale_bf16": [0x3E40, 0x3DC0], "min_bf16": [0x0000, 0x0000]},
+
     # ---- CSR SpMM (spmm_cuda.cu:27-104, reducer.cuh:43-85) -----------------------------------------
     # A = [[1,0,2],[0,0,0],[0,3,0]]; row 1 is empty -> 0 (mean divides by max(count, 1))
     {"op": "spmm", "reduce": "sum", "rowptr": [0, 2, 2, 3], "col": [0, 2, 1], "val": [1, 2, 3],
@@ -108,6 +120,11 @@ CASES = [
     # ---- random projection (ops.py:107-125): X R and X_r R^T ---------------------------------------
     {"op": "rp", "X": [[1, 2, 3], [4, 5, 6]], "R": [[1, 0], [0, -1], [1, 1]],
      "fwd": [[4, 1], [10, 1]], "bwd_of_fwd": [[4, -1, 5], [10, -1, 11]]},
+    # projection then quantisation in one call (ops.py:141-149), 2 bits, noise 0.5, on the product above:
+    # row 0: mn 1, mx 4, scale = fl(1/3) * 3 = 1.0, codes [3, 0]; row 1: mn 1, mx 10, scale = fl(fl(1/9) * 3) =
+    # 0.33333334 (0x3EAAAAAB, bf16 0x3EAB), codes rne([3.0000002, 0]) = [3, 0]; byte d = row 0 | row 1 << 2
+    {"op": "rp_pack", "bits": 2, "X": [[1, 2, 3], [4, 5, 6]], "R": [[1, 0], [0, -1], [1, 1]], "noise": [[HALF] * 2] * 2,
+     "packed": [15, 0, 0], "scale_bf16": [0x3F80, 0x3EAB], "min_bf16": [0x3F80, 0x3F80]},
 ]
 
 if __name__ == "__main__":

@@ -40,7 +40,7 @@ def test_fixture_file_is_what_the_script_writes():
     spec = importlib.util.spec_from_file_location("make_known_answers", path)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
-    assert json.loads(json.dumps(mod.CASES)) == CASES and len({c["op"] for c in CASES}) == 11
+    assert json.loads(json.dumps(mod.CASES)) == CASES and len({c["op"] for c in CASES}) == 13
 
 
 # ------------------------------------------------------------------ oracle side
@@ -120,6 +120,23 @@ def test_oracle_chain(c):
     assert packed.tolist() == c["packed"] and sbf.tolist() == c["scale_bf16"] and mbf.tolist() == c["min_bf16"]
 
 
+@pytest.mark.parametrize("c", pick("bn_relu_dropout_pack"))
+def test_oracle_chain_after_batch_norm(c):
+    x = f32(c["x"])
+    normalised = ((x - f32(c["mean"])[None, :]) * f32(c["mult"])[None, :] + f32(c["shift"])[None, :]).astype(F32)
+    y1, m1 = o.relu_fwd(normalised.reshape(-1))
+    y2, m2 = o.dropout_fwd(y1, c["p"], f32(c["act_noise"]).reshape(-1))
+    packed, _, sbf, mbf, _, _ = o.quantize_activation(y2.reshape(x.shape), c["bits"], f32(c["noise"]))
+    assert np.array_equal(y2.reshape(x.shape), f32(c["y"])) and (m1 & m2).tolist() == c["mask"]
+    assert packed.tolist() == c["packed"] and sbf.tolist() == c["scale_bf16"] and mbf.tolist() == c["min_bf16"]
+
+
+@pytest.mark.parametrize("c", pick("rp_pack"))
+def test_oracle_projection_then_quantisation(c):
+    packed, _, sbf, mbf, _, _ = o.quantize_activation(o.input2rp(f32(c["X"]), f32(c["R"])), c["bits"], f32(c["noise"]))
+    assert packed.tolist() == c["packed"] and sbf.tolist() == c["scale_bf16"] and mbf.tolist() == c["min_bf16"]
+
+
 # ------------------------------------------------------------------ library side
 def dev(a, backend, dtype=None):
     t = torch.from_numpy(np.ascontiguousarray(a))
@@ -181,6 +198,32 @@ def test_library_fused_chain(backend, c):
     assert bytes_equal(sbf, np.array(c["scale_bf16"], np.uint16)) and bytes_equal(mbf, np.array(c["min_bf16"], np.uint16))
     y2, mask2 = extq.relu_dropout_fwd(x, c["p"])
     assert bytes_equal(y2, f32(c["y"])) and mask2.cpu().numpy().view(np.uint32).tolist() == c["mask"]
+
+
+@pytest.mark.parametrize("c", pick("bn_relu_dropout_pack"))
+def test_library_fused_chain_after_batch_norm(backend, c):
+    supply(c["act_noise"], c["noise"])
+    x = dev(f32(c["x"]), backend)
+    vectors = [dev(f32(c[name]), backend) for name in ("mean", "mult", "shift")]
+    y, mask, packed, sbf, mbf = extq.bn_relu_dropout_minmax_pack(x, *vectors, c["p"], c["bits"])
+    assert bytes_equal(y, f32(c["y"])) and mask.cpu().numpy().view(np.uint32).tolist() == c["mask"]
+    assert packed.cpu().numpy().view(np.uint8).tolist() == c["packed"]
+    assert bytes_equal(sbf, np.array(c["scale_bf16"], np.uint16)) and bytes_equal(mbf, np.array(c["min_bf16"], np.uint16))
+
+
+@pytest.mark.parametrize("c", pick("rp_pack"))
+def test_library_projection_then_quantisation(backend, c):
+    supply(c["noise"])
+    R = dev(f32(c["R"]), backend)
+    packed, sbf, mbf = extq.rp_minmax_pack(dev(f32(c["X"]), backend), R, c["bits"])
+    assert packed.cpu().numpy().view(np.uint8).tolist() == c["packed"]
+    assert bytes_equal(sbf, np.array(c["scale_bf16"], np.uint16)) and bytes_equal(mbf, np.array(c["min_bf16"], np.uint16))
+    # and through the public path
+    supply(c["noise"])
+    config.kept_frac, config.activation_compression_bits = 0.5, [c["bits"]]
+    config.rp_matrix_source = lambda D, k, device: R
+    (q, bits, s2, m2), used, shape = ops.project_and_quantize(dev(f32(c["X"]), backend), None)
+    assert used is R and bits == c["bits"] and tuple(shape) == (2, 2) and q.cpu().numpy().view(np.uint8).tolist() == c["packed"]
 
 
 @pytest.mark.parametrize("idx", [torch.int64, torch.int32])
