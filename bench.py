@@ -76,7 +76,7 @@ def run_extras(rows, cols, scale, timeout_s=300):
     the headline figures measured in this process are still printed."""
     import subprocess
     cmd = [sys.executable, "-m", "exact_amd.benchmarks", "extras", "--rows", str(rows), "--cols", str(cols),
-           "--scale", str(scale)]
+           "--scale", str(scale), "--budget", str(timeout_s / 2)]   # no part starts in the second half of the limit
     try:
         res = subprocess.run(cmd, cwd=ROOT, stdout=subprocess.PIPE, timeout=timeout_s, text=True)
     except subprocess.TimeoutExpired:
