@@ -349,6 +349,12 @@ def relu_dropout_fwd(input, p):  # noqa: A002
     return out, mask
 
 
+def _aligned16(t):
+    """t itself, or a copy when its first element is not on a 16-byte boundary
+    (a view into the middle of a buffer): the fused kernels use 16-byte accesses."""
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def relu_dropout_minmax_pack(input, p, bits):  # noqa: A002
     """dropout(relu(input)) and minmax_pack of the result in one pass over
     input[N, G] -> (output, mask, packed int8, scale bf16, min bf16).  Draws
@@ -358,6 +364,7 @@ def relu_dropout_minmax_pack(input, p, bits):  # noqa: A002
     N, G = input.shape
     if not fusable_width(G):
         raise RuntimeError("relu_dropout_minmax_pack needs a row width that is a multiple of 8 and at most 1024")
+    input = _aligned16(input)  # noqa: A001
     dev = input.device
     out = torch.empty_like(input)
     mask = torch.empty(mask_nwords(N * G), dtype=torch.int32, device=dev)
@@ -386,6 +393,7 @@ def bn_relu_dropout_minmax_pack(input, mean, mult, shift, p, bits):  # noqa: A00
             raise RuntimeError(f"The dimension of {name} is not correct!")
     if not fusable_width(G):
         raise RuntimeError("bn_relu_dropout_minmax_pack needs a row width that is a multiple of 8 and at most 1024")
+    input, mean, mult, shift = (_aligned16(t) for t in (input, mean, mult, shift))  # noqa: A001
     dev = input.device
     out = torch.empty_like(input)
     mask = torch.empty(mask_nwords(N * G), dtype=torch.int32, device=dev)

@@ -178,3 +178,24 @@ def test_the_stock_pair_accepts_a_norm_layer():
     bn = torch.nn.BatchNorm1d(8).eval()
     x = torch.randn(5, 8)
     assert torch.equal(ReLUDropout(0.5).eval()(x, norm=bn), F.relu(bn(x)))
+
+
+def test_views_off_a_16_byte_boundary_are_taken(backend):
+    """A bias that lives in the middle of a flat parameter buffer, an input that is a row slice: same results."""
+    config.activation_compression_bits = [2]
+    flat = torch.randn(3 * 16 + 1, device=backend)
+    mean, mult, shift = (flat[1 + 16 * i:1 + 16 * (i + 1)] for i in range(3))
+    assert mean.data_ptr() % 16 != 0
+    big = torch.randn(9, 16, device=backend)
+    x = big.view(-1)[1:1 + 8 * 16].view(8, 16)
+    assert x.data_ptr() % 16 != 0 and x.is_contiguous()
+    _seeded(6)
+    a = extq.bn_relu_dropout_minmax_pack(x, mean, mult, shift, 0.5, 2)
+    _seeded(6)
+    b = extq.bn_relu_dropout_minmax_pack(x.clone(), mean.clone(), mult.clone(), shift.clone(), 0.5, 2)
+    assert all(torch.equal(u, v) for u, v in zip(a, b))
+    _seeded(6)
+    c = extq.relu_dropout_minmax_pack(x, 0.5, 2)
+    _seeded(6)
+    d = extq.relu_dropout_minmax_pack(x.clone(), 0.5, 2)
+    assert all(torch.equal(u, v) for u, v in zip(c, d))
