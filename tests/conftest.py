@@ -22,6 +22,21 @@ def cuda():
 
 
 @pytest.fixture(autouse=True)
+def _seed_per_test(request):
+    """Every test draws the same random inputs whatever ran before it: the
+    global generators (torch CPU and, lazily, GPU; numpy's legacy one) are
+    seeded from the test's id."""
+    import zlib
+
+    import numpy as np
+    import torch
+    seed = zlib.crc32(request.node.nodeid.encode()) & 0x7FFFFFFF
+    torch.manual_seed(seed)
+    np.random.seed(seed)
+    yield
+
+
+@pytest.fixture(autouse=True)
 def _reset_config():
     """Every test starts from the default global config."""
     from exact_amd.conf import QuantizationConfig, config

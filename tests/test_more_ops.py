@@ -92,7 +92,9 @@ def test_leaky_relu_and_elu_layers(backend):
     y2.backward(g2)
     F.elu(x2r, 1.0).backward(g2)
     assert torch.equal(y2, F.elu(x2.detach(), 1.0))
-    assert (x2.grad - x2r.grad).abs().max() < 0.05 and not torch.equal(x2.grad, x2r.grad)
+    # |d/dx elu| differs by at most |g| * exp(max(x, x_hat)) * |x_hat - x| <= |g| * |x_hat - x|, and an 8-bit copy with
+    # bf16 scale / min is within range / 255 + 2^-8 * (|min| + range) of x: below 0.08 for N(0, 1) rows of 32
+    assert ((x2.grad - x2r.grad).abs() <= 0.08 * g2.abs() + 1e-6).all() and not torch.equal(x2.grad, x2r.grad)
     assert torch.equal(layer.eval()(x2.detach()), F.elu(x2.detach(), 1.0))
 
 
