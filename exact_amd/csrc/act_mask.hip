@@ -63,13 +63,13 @@ __device__ __forceinline__ void store4(float* __restrict__ p, int nv, const floa
 template <bool VEC4>
 __device__ __forceinline__ void store4(half_t* __restrict__ p, int nv, const float (&v)[4]) {
   if (VEC4 && nv == 4) {
-    const half4_t a = {static_cast<half_t>(v[0]), static_cast<half_t>(v[1]), static_cast<half_t>(v[2]),
-                       static_cast<half_t>(v[3])};
+    const half4_t a = {to_half(v[0]), to_half(v[1]), to_half(v[2]),
+                       to_half(v[3])};
     __builtin_nontemporal_store(a, reinterpret_cast<half4_t*>(p));
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (i < nv) p[i] = static_cast<half_t>(v[i]);
+      if (i < nv) p[i] = to_half(v[i]);
   }
 }
 

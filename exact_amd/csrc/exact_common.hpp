@@ -93,10 +93,25 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
 
 // ---- fp16 ------------------------------------------------------------------
 // IEEE binary16 with round-to-nearest-even conversions, as at::Half has them.
+//
+// at::Half arithmetic rounds twice: the fp32 operation, then the conversion of
+// its fp32 result.  Written as cast(a * b) the compiler may select
+// v_fma_mixlo_f16, which rounds the exact product ONCE, straight to fp16, and
+// differs in the last bit whenever the fp32 rounding lands on a tie of the
+// fp16 grid.  to_half() therefore first pins its argument in a register as an
+// fp32 value the optimiser cannot look through, so the conversion is always
+// a plain v_cvt_f16_f32 of an already rounded fp32 number.
 using half_t = _Float16;
-__device__ __forceinline__ float round_to_half(float x) { return static_cast<float>(static_cast<half_t>(x)); }
+#ifndef EXACT_VALUE_BARRIER  // the host build of the tests supplies its own constraint letter
+#define EXACT_VALUE_BARRIER(r) asm("" : "+v"(r))
+#endif
+__device__ __forceinline__ half_t to_half(float x) {
+  EXACT_VALUE_BARRIER(x);
+  return static_cast<half_t>(x);
+}
+__device__ __forceinline__ float round_to_half(float x) { return static_cast<float>(to_half(x)); }
 __device__ __forceinline__ uint16_t half_bits(float x) {
-  const half_t h = static_cast<half_t>(x);
+  const half_t h = to_half(x);
   uint16_t b;
   __builtin_memcpy(&b, &h, 2);
   return b;

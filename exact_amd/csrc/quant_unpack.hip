@@ -61,14 +61,14 @@ __device__ __forceinline__ void store_quad_half(half_t* __restrict__ p, int nv, 
   if constexpr (VEC == 4) {
     typedef half_t half4 __attribute__((ext_vector_type(4)));
     if (nv > 0) {
-      const half4 q = {static_cast<half_t>(v[0]), static_cast<half_t>(v[1]), static_cast<half_t>(v[2]),
-                       static_cast<half_t>(v[3])};
+      const half4 q = {to_half(v[0]), to_half(v[1]), to_half(v[2]),
+                       to_half(v[3])};
       __builtin_nontemporal_store(q, reinterpret_cast<half4*>(p));
     }
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (i < nv) __builtin_nontemporal_store(static_cast<half_t>(v[i]), p + i);
+      if (i < nv) __builtin_nontemporal_store(to_half(v[i]), p + i);
   }
 }
 

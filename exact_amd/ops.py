@@ -304,6 +304,8 @@ class qbatch_norm(Function):
         g_in, g_w, g_b = ext_backward_func.native_batch_norm_backward(
             grad_output.contiguous(), x_hat, weight, running_mean, running_var, save_mean, save_invstd, training, eps,
             wanted)
+        # the device routine returns tensors for masked-out outputs too (e.g. without affine parameters)
+        g_in, g_w, g_b = (g if w else None for g, w in zip((g_in, g_w, g_b), wanted))
         return g_in, None, None, g_w, g_b, None, None, None, None
 
 
@@ -530,6 +532,7 @@ class qbn_relu_dropout(Function):
         wanted = [ctx.needs_input_grad[0], ctx.needs_input_grad[3], ctx.needs_input_grad[4]]
         g_in, g_w, g_b = ext_backward_func.native_batch_norm_backward(
             grad_normalised, x_hat, weight, running_mean, running_var, save_mean, save_invstd, True, eps, wanted)
+        g_in, g_w, g_b = (g if w else None for g, w in zip((g_in, g_w, g_b), wanted))
         return g_in, None, None, g_w, g_b, None, None, None, None, None
 
 

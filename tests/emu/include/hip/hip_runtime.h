@@ -44,6 +44,8 @@
 #define __launch_bounds__(...)
 #define __shared__ static thread_local
 #define HIP_DYNAMIC_SHARED(type, var) type* var = reinterpret_cast<type*>(hipemu::dyn_shared());
+// the kernels pin an fp32 value in a register before converting it to fp16; here that is an SSE register
+#define EXACT_VALUE_BARRIER(r) asm("" : "+x"(r))
 
 // ---- vector types ------------------------------------------------------------
 struct float2 { float x, y; };

@@ -19,6 +19,16 @@ def host_randn(shape, seed):
     return torch.randn(shape, generator=g, dtype=torch.float32).numpy()
 
 
+def all_finite_halves():
+    """Every finite fp16 value once (63,488 of them): an exhaustive operand for
+    element-wise fp16 kernels, which therefore contains every input whose fp32
+    result lies on a tie of the fp16 grid -- the inputs on which rounding the
+    exact result once differs from rounding the fp32 result a second time."""
+    bits = np.arange(1 << 16, dtype=np.uint16)
+    v = bits.view(np.float16)
+    return v[np.isfinite(v)].copy()
+
+
 class FixedNoise:
     """config.noise_source that hands out pre-made tensors in call order."""
 

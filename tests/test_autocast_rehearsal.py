@@ -1,6 +1,6 @@
 """The autocast (fp16) training path, rehearsed on the CPU in a separate
 process (tests/autocast_rehearsal.py explains how); the GPU run of the same
-path is tests/test_y_half_layers.py::test_training_step_under_autocast."""
+path is tests/test_zz_half_layers.py::test_training_step_under_autocast."""
 import os
 import subprocess
 import sys

@@ -61,3 +61,20 @@ def test_mask_kernels_f16(n):
             wy, wm = oh.dropout_fwd(x, 0.3, un, relu=relu)
             assert np.array_equal(u16(y), u16(wy)) and np.array_equal(m, wm)
             assert np.array_equal(u16(e.mask_bwd_f16("dropout", g, m, 0.3)), u16(oh.dropout_bwd(g, wm, 0.3)))
+
+
+def test_mask_kernels_f16_round_twice_on_every_operand():
+    """All finite fp16 values through the scaling kernels, at constants for which
+    rounding once and rounding twice differ (tests/test_oracle_half.py)."""
+    from gpu_util import all_finite_halves
+    x = all_finite_halves()
+    ones = np.ones(x.size, F32)
+    y, m = e.leaky_relu_fwd_f16(x, 0.1)
+    wy, wm = oh.leaky_relu_fwd(x, 0.1)
+    assert np.array_equal(u16(y), u16(wy)) and np.array_equal(m, wm)
+    assert np.array_equal(u16(e.mask_bwd_f16("leaky", x, np.zeros_like(m), 0.1)),
+                          u16(oh.leaky_relu_bwd(x, np.zeros_like(wm), 0.1)))
+    y, m = e.dropout_fwd_f16(x, 0.4, ones, 0, 0)
+    wy, wm = oh.dropout_fwd(x, 0.4, ones)
+    assert np.array_equal(u16(y), u16(wy)) and np.array_equal(m, wm)
+    assert np.array_equal(u16(e.mask_bwd_f16("dropout", x, m, 0.4)), u16(oh.dropout_bwd(x, wm, 0.4)))

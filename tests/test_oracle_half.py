@@ -93,3 +93,59 @@ def test_mask_ops_match_torch_half():
     y1, m1 = oh.relu_fwd(x)
     y3, m3 = oh.dropout_fwd(y1, 0.3, u)
     assert np.array_equal(y2.view(np.uint16), y3.view(np.uint16)) and np.array_equal(m2, m1 & m3)
+
+
+def _once(exact64):
+    """fp64 (exact or correctly rounded) result -> fp16 in ONE rounding."""
+    with np.errstate(over="ignore"):
+        return np.asarray(exact64, np.float64).astype(F16)
+
+
+def test_dropout_rounds_twice_and_the_layer_test_inputs_tell_the_difference():
+    """at::Half arithmetic rounds the fp32 product and then converts it to
+    fp16.  A kernel that rounds the exact product once (what a fused
+    multiply-and-convert instruction does) differs on inputs whose fp32 result
+    is a tie of the fp16 grid.  The inputs of the layer test (seed 0, 100 x 48,
+    p = 0.4) must contain such elements, so that test can tell the two apart."""
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal((100, 48)) * 3).astype(F16).reshape(-1)
+    rng.standard_normal((100, 48))
+    u = rng.random((100, 48), dtype=F32).reshape(-1)
+    y, _ = oh.dropout_fwd(x, 0.4, u)
+    pinv = F32(1.0 / (1.0 - float(F32(0.4))))
+    keep = u > F32(0.4)
+    once = _once(x.astype(np.float64) * keep * float(pinv))        # 11-bit x 24-bit: exact in fp64
+    differ = (y.view(np.uint16) != once.view(np.uint16)) & (y != 0)
+    assert differ.sum() == 185
+    # and torch's fp16 CPU arithmetic agrees with the oracle on every one of them
+    want = (torch.from_numpy(x).float() * torch.from_numpy(keep).float() * float(pinv)).half().numpy()
+    assert np.array_equal(y.view(np.uint16), want.view(np.uint16))
+
+
+def test_every_half_operand_separates_one_rounding_from_two():
+    """The exhaustive operand (all finite fp16 values) used by the kernel tests
+    contains double-rounding cases for each element-wise fp16 operation -- at
+    the constants those tests use (slope 0.1, p = 0.4).  Slope 0.2 and p = 0.3
+    have no such case over the whole fp16 range, so passing with them shows
+    nothing about the rounding."""
+    from gpu_util import all_finite_halves
+    x = all_finite_halves()
+    ones = np.ones(x.size, F32)
+    neg = ~(x > 0)
+
+    def leaky_cases(slope):
+        y, _ = oh.leaky_relu_fwd(x, slope)
+        return (y[neg].view(np.uint16) != _once(x[neg].astype(np.float64) * float(F32(slope))).view(np.uint16)).sum()
+
+    def dropout_cases(p):
+        y, m = oh.dropout_fwd(x, p, ones)
+        pinv = F32(1.0 / (1.0 - float(F32(p))))
+        p1m = F32(1.0 - float(F32(p)))
+        fwd = (y.view(np.uint16) != _once(x.astype(np.float64) * float(pinv)).view(np.uint16)).sum()
+        bwd = (oh.dropout_bwd(x, m, p).view(np.uint16) != _once(x.astype(np.float64) / float(p1m)).view(np.uint16)).sum()
+        return fwd, bwd
+
+    assert leaky_cases(0.1) > 50 and leaky_cases(0.2) == 0
+    fwd, bwd = dropout_cases(0.4)
+    assert fwd > 1000 and bwd > 1000
+    assert dropout_cases(0.3) == (0, 0)

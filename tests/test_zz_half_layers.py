@@ -16,7 +16,7 @@ from exact_amd.cpp_extension import quantization as extq
 from exact_amd.cpp_extension import spmm as ext_spmm
 from exact_amd.models import GCN
 from exact_amd.sparse import SparseTensor, gcn_norm
-from gpu_util import FixedNoise, bytes_equal
+from gpu_util import FixedNoise, all_finite_halves, bytes_equal
 
 F16, F32 = np.float16, np.float32
 
@@ -74,6 +74,26 @@ def test_mask_layers_fp16(backend):
         assert y.dtype == torch.float16 and bytes_equal(y, wy)
         assert bytes_equal(xt.grad, oh.dropout_bwd(g.reshape(-1), wm, 0.4))
         assert ops.take_compressed(y) is None               # the one-pass quantiser is fp32 only
+
+
+def test_mask_layers_fp16_round_twice_on_every_operand(backend):
+    """Every finite fp16 value through LeakyReLU (slope 0.1) and dropout
+    (p = 0.4), forward and backward: constants at which a kernel that rounds
+    the exact product once differs from at::Half's two roundings in thousands
+    of these operands (tests/test_oracle_half.py)."""
+    x = all_finite_halves()
+    ones = np.ones(x.size, F32)
+    xt = torch.from_numpy(x).to(backend).requires_grad_()
+    y = exact.QLeakyReLU(0.1).train()(xt)
+    y.backward(torch.from_numpy(-np.abs(x)).to(backend))     # gradient operand on the scaled side as well
+    wy, wm = oh.leaky_relu_fwd(x, 0.1)
+    assert bytes_equal(y, wy) and bytes_equal(xt.grad, oh.leaky_relu_bwd(-np.abs(x), wm, 0.1))
+    xt.grad = None
+    config.noise_source = FixedNoise([torch.from_numpy(ones)])
+    y = exact.QDropout(0.4).train()(xt)
+    y.backward(xt.detach())
+    wy, wm = oh.dropout_fwd(x, 0.4, ones)
+    assert bytes_equal(y, wy) and bytes_equal(xt.grad, oh.dropout_bwd(x, wm, 0.4))
 
 
 def test_linear_and_sparse_products_fp16(backend):
