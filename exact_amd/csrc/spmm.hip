@@ -22,11 +22,10 @@
 namespace exact {
 
 constexpr int kChunk = 64;  // entries per wavefront == lanes per wavefront
-constexpr int kGather = 8;  // X rows in flight per lane
+constexpr int kGather = 8;  // X rows in flight per lane (4 and 16 measure the same)
 constexpr int kXcds = 8;    // accelerator complex dies of an MI355X, each with its own L2
 
 template <int VEC> struct Vec;
-template <> struct Vec<4> { using T = float4; };
 template <> struct Vec<2> { using T = float2; };
 template <> struct Vec<1> { using T = float; };
 
@@ -235,13 +234,20 @@ int exact_spmm_csr_f32(const void* rowptr, const void* col, const float* val, in
     hipLaunchKernelGGL((spmm_zero_rows_kernel<int64_t>), zgrid, dim3(kBlock), 0, s,
                        static_cast<const int64_t*>(rowptr), M, K, out);
   if (nnz > 0) {
-    const int vec = (K % 4 == 0 && al(X, 16) && al(out, 16)) ? 4 : (K % 2 == 0 && al(X, 8) && al(out, 8)) ? 2 : 1;
+    // Column tile of one wavefront = 64 * vec columns.  Measured on power-law
+    // graphs of 170k to 2.4M rows: 8-byte gathers (128-column tiles) beat 16-byte
+    // ones (256-column tiles) by 6 to 40 % at every width from 100 to 600 -- twice
+    // as many wavefronts share the same gathers -- so 16-byte gathers are not
+    // used; rows of at most 64 columns take 4-byte gathers (one tile, more lanes
+    // busy than with wider ones).
+    const int vec = (K > 64 && K % 2 == 0 && al(X, 8) && al(out, 8)) ? 2 : 1;
+    if ((K + kWave * vec - 1) / (kWave * vec) > 65535) return EXACT_E_SHAPE;  // grid.y limit
 #define EXACT_SPMM_GO(I, V) \
   spmm_dispatch<I, V>(static_cast<const I*>(rowptr), static_cast<const I*>(col), val, X, M, nnz, K, reduce, out, s)
     if (idx_bytes == 4) {
-      if (vec == 4) EXACT_SPMM_GO(int32_t, 4); else if (vec == 2) EXACT_SPMM_GO(int32_t, 2); else EXACT_SPMM_GO(int32_t, 1);
+      if (vec == 2) EXACT_SPMM_GO(int32_t, 2); else EXACT_SPMM_GO(int32_t, 1);
     } else {
-      if (vec == 4) EXACT_SPMM_GO(int64_t, 4); else if (vec == 2) EXACT_SPMM_GO(int64_t, 2); else EXACT_SPMM_GO(int64_t, 1);
+      if (vec == 2) EXACT_SPMM_GO(int64_t, 2); else EXACT_SPMM_GO(int64_t, 1);
     }
 #undef EXACT_SPMM_GO
   }

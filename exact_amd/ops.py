@@ -268,15 +268,17 @@ class qlinear(Function):
     def backward(ctx, grad_output):
         kept, ctx.kept = ctx.kept, None
         if kept.randmat is None:
-            grads = ext_backward_func.linear_backward(grad_output, kept.restore(), ctx.weight, ctx.bias)
+            grads = ext_backward_func.linear_backward(grad_output, kept.restore(), ctx.weight, ctx.bias,
+                                                      ctx.needs_input_grad[0])
         else:
             # dW = dY^T (X_r R^T) = (dY^T X_r) R^T: the [N, D] decompressed input of
             # the reference (ops.py:163-165) is never formed; only the order in
             # which fp32 sums are taken differs.
             x_r = dequantize_activation(kept.quantized, kept.stored_shape)
-            grad_input = grad_output.mm(ctx.weight)
+            grad_input = grad_output.mm(ctx.weight) if ctx.needs_input_grad[0] else None
             grad_weight = grad_output.t().mm(x_r).mm(kept.randmat.t())
-            grads = (grad_input, grad_weight, grad_output.sum(0) if ctx.bias is not None else None)
+            grads = (grad_input, grad_weight,
+                     ext_backward_func.column_sums(grad_output) if ctx.bias is not None else None)
         empty_cache(config.empty_cache_threshold)
         return (*grads, None, None, None, None)
 

@@ -176,6 +176,13 @@ int exact_elu_bwd_f32(const float *dy, const float *x, float alpha, int64_t n,
 int exact_elu_bwd_f16(const uint16_t *dy, const uint16_t *x, float alpha, int64_t n,
                       uint16_t *dx, void *stream);
 
+/* Column sums of a row-major [N, K] fp32 matrix, out[k] = sum_n x[n, k], K <= 8192,
+ * x 16-byte aligned.  Replaces `grad_output.sum(0)`, the bias gradient of
+ * linear_backward (backward_func.cc:90-91), whose library reduction is far off
+ * the memory roofline for narrow matrices.  fp32 atomics: the summation order
+ * is not fixed. */
+int exact_colsum_f32(const float *x, int64_t N, int64_t K, float *out, void *stream);
+
 /* Fused epilogues (no single counterpart in the reference: each replaces a
  * chain of its calls with one pass over the data, bit-identical to the chain).
  *

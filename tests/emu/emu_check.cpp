@@ -420,6 +420,20 @@ static void check_half(int64_t N, int64_t G, int bits, std::mt19937& rng) {
   CHECK(rc == 0, "f16 mask entry points rc=%d", rc);
 }
 
+static void check_colsum(int64_t N, int64_t K, std::mt19937& rng) {
+  std::uniform_int_distribution<int> id(-8, 8);
+  Buf<float> x(static_cast<size_t>(N * K)), out(static_cast<size_t>(K));
+  std::vector<double> want(static_cast<size_t>(K), 0.0);
+  for (int64_t i = 0; i < N * K; ++i) {
+    x[i] = static_cast<float>(id(rng));
+    want[static_cast<size_t>(i % K)] += x[i];
+  }
+  const int rc = exact_colsum_f32(x.p, N, K, out.p, nullptr);
+  CHECK(rc == 0, "colsum rc %d N=%lld K=%lld", rc, (long long)N, (long long)K);
+  for (int64_t k = 0; k < K; ++k)
+    CHECK(out[k] == static_cast<float>(want[static_cast<size_t>(k)]), "colsum N=%lld K=%lld col %lld", (long long)N, (long long)K, (long long)k);
+}
+
 int main(int argc, char** argv) {
   std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
@@ -463,6 +477,9 @@ int main(int argc, char** argv) {
   for (auto& f : hs)
     for (int bits : {1, 2, 4, 8}) check_half(f[0], f[1], bits, rng);
   std::printf("fp16 entry points ok (failures so far %d)\n", g_fail);
+  const int64_t cs[][2] = {{1, 1}, {3, 5}, {7, 47}, {1000, 41}, {4099, 47}, {513, 256}, {33, 602}, {5, 8192}, {20000, 3}};
+  for (auto& c : cs) check_colsum(c[0], c[1], rng);
+  std::printf("column sums ok (failures so far %d)\n", g_fail);
   if (mode == "large" || mode == "full") {
     for (int bits : {1, 2, 4, 8}) check_quant(20011, 256, bits, bits == 4, rng);
     check_quant(3001, 1024, 2, false, rng);

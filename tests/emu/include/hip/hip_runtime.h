@@ -64,6 +64,10 @@ typedef int hipError_t;
 typedef void* hipStream_t;
 constexpr hipError_t hipSuccess = 0;
 static inline hipError_t hipGetLastError() { return hipSuccess; }
+// one emulated device; a small CU count keeps the persistent kernels' grids small here
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 63 };
+static inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+static inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 2; return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "hip emulator: no error"; }
 
 using std::max;

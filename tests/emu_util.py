@@ -370,3 +370,16 @@ def spmm_rowwise(rowptr, col, val, X, reduce, idx=np.int64, guard=16):
     assert rc == 0, rc
     assert (out[M * K:] == np.float32(-777.0)).all()
     return out[:M * K].reshape(M, K)
+
+
+def colsum(x, guard=8, expect_rc=0):
+    """exact_colsum_f32 -> fp32 [K]."""
+    x = f32(x)
+    N, K = x.shape
+    out = np.full(K + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_colsum_f32(p(x), N, K, p(out), None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (out[K:] == np.float32(-777.0)).all()
+    return out[:K]

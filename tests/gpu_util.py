@@ -79,3 +79,22 @@ class SeededNoise:
 
     def rp_matrix_source(self, D, k, device):
         return self.rademacher(D, k, device)
+
+
+def powerlaw_csr(n, raw_edges, seed, alpha=2.1):
+    """Host-side power-law graph of the benchmark's kind (out-degree with a
+    Pareto tail of exponent alpha, uniformly random targets, symmetrised,
+    de-duplicated, no self loops) as a scipy CSR pattern matrix."""
+    import scipy.sparse as sp
+    rng = np.random.default_rng(seed)
+    raw = np.minimum(rng.random(n).clip(1e-9) ** (-1.0 / (alpha - 1.0)), max(64, n // 16))
+    deg = np.clip(np.rint(raw * (raw_edges / raw.sum())), 1, max(64, n // 16)).astype(np.int64)
+    src = np.repeat(np.arange(n), deg)
+    dst = rng.integers(0, n, src.size)
+    keep = src != dst
+    src, dst = src[keep], dst[keep]
+    A = sp.coo_matrix((np.ones(2 * src.size, np.float32), (np.concatenate([src, dst]), np.concatenate([dst, src]))),
+                      shape=(n, n)).tocsr()
+    A.data[:] = 1.0
+    A.sort_indices()
+    return A

@@ -15,7 +15,7 @@ from exact_amd import ops
 from exact_amd.conf import config
 from exact_amd.models import GCN, SAGE
 from exact_amd.sparse import SparseTensor, gcn_norm
-from gpu_util import SeededNoise
+from gpu_util import SeededNoise, powerlaw_csr
 
 
 def tol(device):
@@ -209,6 +209,79 @@ def test_gcn_training_loss_tracks_oracle_for_20_steps(backend):
         assert abs(loss.item() - loss_o.item()) < 1e-3, (step, loss.item(), loss_o.item())
     assert np.isfinite(loss.item())
     print(f"max |loss - oracle loss| over {steps} steps: {worst:.2e}")
+
+
+def test_deep_gcn_training_loss_tracks_oracle_for_20_steps(backend):
+    """The full-batch GCN benchmark configuration at a size the oracle finishes
+    in about a minute: 3 layers 128 -> 256 -> 256 -> 40 with BatchNorm, ReLU
+    and dropout 0.5, INT2, kept_frac 1, on a symmetrised power-law graph with
+    self loops and symmetric normalisation (mem_speed_bench/models/gcn.py:54-61,
+    arxiv/conf/gcn.yaml:5-9, the loop of arxiv/train_full_batch.py:256-266 of
+    the reference).  20 optimiser steps; the loss stays within 1e-3 of the
+    oracle model's at every step."""
+    n = 20000 if backend.type == "cuda" else 1500
+    feat, hidden, classes, steps = 128, 256, 40, 20
+    A = powerlaw_csr(n, int(n * 6.85), 2)
+    adj = gcn_norm(SparseTensor.from_scipy(A).set_value(None), add_self_loops=True)
+    rowptr, col, value = adj.csr()
+    graph = om.Graph(rowptr.numpy(), col.numpy(), value.numpy())
+    adj = adj.to(backend).fill_cache_()
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(n, feat, generator=g)
+    labels = torch.randint(0, classes, (n,), generator=g)
+    train_idx = torch.randperm(n, generator=g)[: n // 2]
+    torch.manual_seed(7)
+    model = exact.QModule(GCN(feat, hidden, classes, 3, dropout=0.5, batch_norm=True)).to(backend).train()
+    params = _params_of_gcn(model)
+    bn_state = [(b.running_mean.detach().cpu().clone(), b.running_var.detach().cpu().clone()) for b in model.model.bns]
+    other = wire_noise(23)
+    c = om.Ctx(2, 1.0, other.noise, None)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    opt_o = torch.optim.SGD(_flat(params), lr=0.05)
+    xd, yd, idx = x.to(backend), labels.to(backend), train_idx.to(backend)
+    worst = 0.0
+    for step in range(steps):
+        opt.zero_grad()
+        loss = F.nll_loss(F.log_softmax(model(xd, adj)[idx], dim=-1), yd[idx])
+        loss.backward()
+        opt.step()
+        opt_o.zero_grad()
+        out_o = om.gcn_forward(c, params, graph, x, 0.5, True, bn_state)
+        loss_o = F.nll_loss(F.log_softmax(out_o[train_idx], dim=-1), labels[train_idx])
+        loss_o.backward()
+        opt_o.step()
+        worst = max(worst, abs(loss.item() - loss_o.item()))
+        assert abs(loss.item() - loss_o.item()) < 1e-3, (step, loss.item(), loss_o.item())
+    print(f"max |loss - oracle loss| over {steps} steps: {worst:.2e}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["cfg3_gcn_int2", "cfg4_sage_int2_rp0.125", "cfg5_sage_int1_rp0.25"])
+def test_full_size_training_steps_are_finite_and_learn(cuda, name):
+    """The three full-batch benchmark configurations at their full size: a few
+    epochs of the reference's loop; every loss is finite and the loss falls."""
+    from exact_amd import benchmarks as B
+    losses = []
+    real = B.train_epochs
+
+    def spy(model, x, adj, labels, train_idx, epochs, warmup, lr=0.01):
+        opt = torch.optim.Adam(model.parameters(), lr=lr)
+        model.train()
+        for _ in range(epochs):
+            opt.zero_grad()
+            loss = F.nll_loss(F.log_softmax(model(x, adj)[train_idx], dim=-1), labels[train_idx])
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+            assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+        return 1.0, losses[-1]
+
+    B.train_epochs = spy
+    try:
+        B.epoch_benchmark(name, cuda, lambda *a: None, epochs=4, warmup=0)
+    finally:
+        B.train_epochs = real
+    assert len(losses) == 4 and all(np.isfinite(l) for l in losses) and losses[-1] < losses[0]
 
 
 @pytest.mark.parametrize("kept_frac,bits", [(0.125, 2), (0.25, 1)])

@@ -527,3 +527,39 @@ def test_deterministic_spmm_switch(backend):
             torch.use_deterministic_algorithms(False)
         assert np.array_equal(y.detach().cpu().numpy().view(np.uint32), want.view(np.uint32))
         assert np.array_equal(x.grad.cpu().numpy().view(np.uint32), want_bw.view(np.uint32))
+
+
+@pytest.mark.parametrize("N,K", [(1, 1), (3, 5), (7, 47), (1000, 41), (4099, 47), (513, 256), (2050, 100), (33, 602),
+                                 (5, 8192), (40000, 3)])
+def test_column_sum_kernel_counts_every_element_once(N, K):
+    """exact_colsum_f32 on small integers, whose fp32 sums are exact whatever the
+    order: any element missed, counted twice or added to the wrong column shows."""
+    rng = np.random.default_rng(N * 7 + K)
+    x = rng.integers(-8, 9, (N, K)).astype(np.float32)
+    got = e.colsum(x)
+    assert np.array_equal(got, x.astype(np.float64).sum(0).astype(np.float32))
+    y = rng.standard_normal((N, K)).astype(np.float32)
+    want = y.astype(np.float64).sum(0)
+    assert np.allclose(e.colsum(y), want, rtol=0, atol=1e-6 * np.abs(y).astype(np.float64).sum(0).max() + 1e-30)
+
+
+def test_column_sum_limits():
+    assert e.colsum(np.zeros((2, 8193), np.float32), expect_rc=-3) is None
+    assert e.colsum(np.zeros((0, 5), np.float32)).tolist() == [0.0] * 5
+
+
+def test_bias_gradient_goes_through_the_column_sum_kernel(backend):
+    """linear_backward's grad_output.sum(0) (backward_func.cc:90-91) for a tall
+    fp32 matrix: same numbers as the framework's reduction to rounding."""
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator().manual_seed(5)
+    for N, K in ((5000, 47), (4096, 256), (6001, 41)):
+        dy = torch.randn(N, K, generator=g).to(backend)
+        got = bf.column_sums(dy)
+        want = dy.double().sum(0)
+        assert got.dtype == torch.float32 and got.shape == (K,)
+        assert (got.double() - want).abs().max().item() <= 1e-6 * dy.abs().double().sum(0).max().item()
+        ints = torch.randint(-8, 9, (N, K), generator=g).float().to(backend)
+        assert torch.equal(bf.column_sums(ints), ints.sum(0))
+    small = torch.randn(10, 3).to(backend)
+    assert torch.equal(bf.column_sums(small), small.sum(0))       # short matrices keep the framework's reduction
