@@ -35,6 +35,7 @@ SIGNATURES = {
     "exact_dropout_fwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_u64, _c_u64, _c_f32, _c_i64, _c_ptr, _c_ptr, _c_ptr]),
     "exact_dropout_bwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_spmm_csr_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
+    "exact_spmm_csr_strided_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_i64, _c_ptr]),
     "exact_spmm_csr_rowwise_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
     "exact_spmm_csr_minmax_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr]),
     "exact_sddmm_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
@@ -58,6 +59,8 @@ SIGNATURES = {
     "exact_dropout_bwd_f16": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_elu_bwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_colsum_f32": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr]),
+    "exact_col_moments_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr]),
+    "exact_bn_backward_reduce_f32": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr]),
     "exact_elu_bwd_f16": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_rp_fwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_rp_bwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),

@@ -15,8 +15,8 @@ def column_sums(matrix):
     fix no summation order, so deterministic mode and everything else keep the
     framework's reduction."""
     usable = (matrix.dim() == 2 and matrix.dtype == torch.float32 and _checks.on_device(matrix)
-              and matrix.is_contiguous() and 0 < matrix.shape[1] <= 8192 and matrix.shape[0] >= 4096
-              and matrix.data_ptr() % 16 == 0 and not torch.are_deterministic_algorithms_enabled())
+              and matrix.is_contiguous() and 0 < matrix.shape[1] <= 256 and matrix.shape[0] >= 4096
+              and not torch.are_deterministic_algorithms_enabled())
     if not usable:
         return matrix.sum(0)
     out = torch.empty(matrix.shape[1], dtype=torch.float32, device=matrix.device)
@@ -24,6 +24,28 @@ def column_sums(matrix):
                                      _checks.stream_ptr(matrix))
     _lib.check(rc, "column_sums")
     return out
+
+
+def batch_statistics(matrix):
+    """(biased variance, mean) of every column of a 2-D tensor, what
+    torch.var_mean(matrix, dim=0, unbiased=False) returns.  Tall fp32 device
+    matrices of at most 256 columns take the library's one-pass kernel (moments
+    centred on the mean of the first 256 rows, close enough to the column mean
+    that the difference of the two moments loses no digits); everything else
+    the framework's reduction."""
+    usable = (matrix.dim() == 2 and matrix.dtype == torch.float32 and matrix.is_cuda and matrix.is_contiguous()
+              and 0 < matrix.shape[1] <= 256 and matrix.shape[0] >= 4096
+              and not torch.are_deterministic_algorithms_enabled())
+    if not usable:
+        return torch.var_mean(matrix, dim=0, unbiased=False)
+    N, K = matrix.shape
+    center = matrix[:256].mean(0)
+    sums = torch.empty((2, K), dtype=torch.float32, device=matrix.device)
+    rc = _lib.lib().exact_col_moments_f32(_checks.ptr(matrix), _checks.ptr(center), N, K, _checks.ptr(sums[0]),
+                                          _checks.ptr(sums[1]), _checks.stream_ptr(matrix))
+    _lib.check(rc, "batch_statistics")
+    shift = sums[0] / N
+    return (sums[1] / N - shift * shift).clamp_(min=0.0), center + shift
 
 
 def linear_backward(grad_output, input, weight, bias, need_input_grad=True):  # noqa: A002
@@ -41,8 +63,38 @@ def native_batch_norm(input, weight, bias, running_mean, running_var, training, 
 
 def native_batch_norm_backward(grad_out, input, weight, running_mean, running_var, save_mean, save_invstd,  # noqa: A002
                                train, eps, output_mask):
-    return torch.ops.aten.native_batch_norm_backward(grad_out, input, weight, running_mean, running_var,
-                                                     save_mean, save_invstd, train, eps, list(output_mask))
+    """at::native_batch_norm_backward as re-exported by backward_func.cc:99-104.
+    For a tall fp32 [N, K <= 256] training-mode batch on the device, its two
+    column reductions (sum of dy, sum of dy * (x - mean)) run in the library's
+    one-pass kernel -- the framework's reduction kernel reads the same two
+    matrices at a tenth of the memory bandwidth -- and the element-wise half is
+    the framework's batch_norm_backward_elemt, which computes
+      dx = (dy - sum_dy / N - (x - mean) * invstd^2 * sum_dy_xmu / N) * invstd * weight
+    exactly as the one-call routine does."""
+    fast = (train and grad_out.dim() == 2 and grad_out.is_cuda and grad_out.dtype == torch.float32
+            and input.dtype == torch.float32 and grad_out.is_contiguous() and input.is_contiguous()
+            and grad_out.shape[0] >= 4096 and 0 < grad_out.shape[1] <= 256 and grad_out.shape == input.shape
+            and save_mean is not None and save_invstd is not None and save_mean.dtype == torch.float32
+            and not torch.are_deterministic_algorithms_enabled())
+    if not fast:
+        return torch.ops.aten.native_batch_norm_backward(grad_out, input, weight, running_mean, running_var,
+                                                         save_mean, save_invstd, train, eps, list(output_mask))
+    N, K = grad_out.shape
+    mean = save_mean.contiguous()
+    sums = torch.empty((2, K), dtype=torch.float32, device=grad_out.device)
+    rc = _lib.lib().exact_bn_backward_reduce_f32(_checks.ptr(grad_out), _checks.ptr(input), _checks.ptr(mean), N, K,
+                                                 _checks.ptr(sums[0]), _checks.ptr(sums[1]), _checks.stream_ptr(grad_out))
+    _lib.check(rc, "native_batch_norm_backward")
+    sum_dy, sum_dy_xmu = sums[0], sums[1]
+    grad_input = grad_weight = grad_bias = None
+    if output_mask[0]:
+        count = torch.full((1,), N, dtype=torch.int32, device=grad_out.device)
+        grad_input = torch.batch_norm_backward_elemt(grad_out, input, mean, save_invstd, weight, sum_dy, sum_dy_xmu, count)
+    if output_mask[1]:
+        grad_weight = sum_dy_xmu * save_invstd
+    if output_mask[2]:
+        grad_bias = sum_dy
+    return grad_input, grad_weight, grad_bias
 
 
 def _elu_backward_cuda(grad_output, data, alpha):

@@ -52,16 +52,40 @@ def spmm_csr(rowptr, col, value, mat, reduce):
     if rowptr.dtype != col.dtype:
         wide = torch.int64 if torch.int64 in (rowptr.dtype, col.dtype) else torch.int32
         rowptr, col = rowptr.to(wide), col.to(wide)
-    rowptr, col, mat = rowptr.contiguous(), col.contiguous(), mat.contiguous()
+    rowptr, col = rowptr.contiguous(), col.contiguous()
     M = rowptr.numel() - 1
     n_cols, K = mat.shape
     out = torch.empty((M, K), dtype=mat.dtype, device=mat.device)
     reproducible = config.deterministic_spmm or torch.are_deterministic_algorithms_enabled()
-    kernel = _lib.lib().exact_spmm_csr_rowwise_f32 if reproducible else _lib.lib().exact_spmm_csr_f32
-    rc = kernel(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat),
-                M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out), _checks.stream_ptr(mat))
+    if reproducible:
+        mat = mat.contiguous()
+        rc = _lib.lib().exact_spmm_csr_rowwise_f32(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat),
+                                                   M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out),
+                                                   _checks.stream_ptr(mat))
+    else:
+        mat = _aligned_rows(mat, col.numel())
+        rc = _lib.lib().exact_spmm_csr_strided_f32(ptr(rowptr), ptr(col), ptr(value), rowptr.element_size(), ptr(mat),
+                                                   mat.stride(0), M, n_cols, K, col.numel(), REDUCE[reduce], ptr(out), K,
+                                                   _checks.stream_ptr(mat))
     _lib.check(rc, f"spmm_{reduce}")
     return out
+
+
+def _aligned_rows(mat, nnz):
+    """The dense operand as the kernel wants it: unit column stride, any row
+    stride.  Wide rows whose length is not a multiple of 128 bytes are copied
+    into rows padded to one when the graph is dense enough to pay for the copy:
+    a wavefront gathers 512-byte pieces of a row, and an unaligned piece
+    straddles five 128-byte lines instead of four (602 columns, average degree
+    100: 8.9 ms -> 7.2 ms per product for a 0.2 ms copy)."""
+    if mat.stride(1) != 1 or mat.stride(0) < mat.shape[1]:
+        mat = mat.contiguous()
+    n_cols, K = mat.shape
+    if K > 128 and K % 32 != 0 and mat.stride(0) == K and n_cols > 0 and nnz >= 16 * n_cols:
+        padded = torch.empty((n_cols, (K + 31) // 32 * 32), dtype=mat.dtype, device=mat.device)
+        padded[:, :K].copy_(mat)
+        return padded[:, :K]
+    return mat
 
 
 def _missing(name):

@@ -15,7 +15,8 @@
 //   * a row that lies wholly inside one chunk is accumulated in CSR order and
 //     written with a plain store; a row that straddles chunks is accumulated
 //     per chunk and combined with fp32 atomic adds into rows that a small
-//     pre-pass has zeroed (the same pre-pass zeroes empty rows).
+//     pre-pass has zeroed (the same pre-pass zeroes empty rows); for the mean a
+//     small post-pass divides those rows' totals by the row length.
 
 #include "exact_common.hpp"
 
@@ -56,7 +57,7 @@ __device__ __forceinline__ int64_t readlane_i64(int64_t v, int lane) {
 // plain store: it is empty, or it spans more than one chunk.
 template <typename I>
 __global__ __launch_bounds__(kBlock) void spmm_zero_rows_kernel(const I* __restrict__ rowptr, int64_t M,
-                                                                int64_t K, float* __restrict__ out) {
+                                                                int64_t K, int64_t ldo, float* __restrict__ out) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t base = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + (threadIdx.x >> 6)) * kWave;
   const int64_t r = base + lane;
@@ -69,8 +70,33 @@ __global__ __launch_bounds__(kBlock) void spmm_zero_rows_kernel(const I* __restr
   while (todo) {
     const int l = __builtin_ctzll(todo);
     todo &= todo - 1;
-    float* dst = out + (base + l) * K;
+    float* dst = out + (base + l) * ldo;
     for (int64_t c = lane; c < K; c += kWave) dst[c] = 0.f;
+  }
+}
+
+// Mean aggregation, rows that span more than one chunk: the chunk kernel has
+// added up their partial sums; divide by the row length (reducer.cuh:75-76).
+template <typename I>
+__global__ __launch_bounds__(kBlock) void spmm_mean_finish_kernel(const I* __restrict__ rowptr, int64_t M,
+                                                                  int64_t K, int64_t ldo, float* __restrict__ out) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t base = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + (threadIdx.x >> 6)) * kWave;
+  const int64_t r = base + lane;
+  bool split = false;
+  float len = 1.f;
+  if (r < M) {
+    const int64_t rs = rowptr[r], re = rowptr[r + 1];
+    split = (re > rs) && (rs / kChunk != (re - 1) / kChunk);
+    len = static_cast<float>(re - rs);
+  }
+  uint64_t todo = __ballot(split);
+  while (todo) {
+    const int l = __builtin_ctzll(todo);
+    todo &= todo - 1;
+    const float d = readlane_f(len, l);
+    float* dst = out + (base + l) * ldo;
+    for (int64_t c = lane; c < K; c += kWave) dst[c] = dst[c] / d;
   }
 }
 
@@ -79,7 +105,7 @@ __global__ __launch_bounds__(kBlock) void spmm_chunk_kernel(const I* __restrict_
                                                             const I* __restrict__ col,
                                                             const float* __restrict__ val,
                                                             const float* __restrict__ X, int64_t M,
-                                                            int64_t nnz, int64_t K,
+                                                            int64_t nnz, int64_t K, int64_t ldx, int64_t ldo,
                                                             float* __restrict__ out) {
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
@@ -134,16 +160,18 @@ __global__ __launch_bounds__(kBlock) void spmm_chunk_kernel(const I* __restrict_
 
   auto flush = [&]() {
     if (row_end > row_start && kok) {
-      float res[VEC];
-#pragma unroll
-      for (int c = 0; c < VEC; ++c)
-        res[c] = MEAN ? acc[c] / static_cast<float>(row_end - row_start) : acc[c];  // reducer.cuh:75-76
-      float* dst = out + r * K + kcol;
+      float* dst = out + r * ldo + kcol;
       if (row_start >= e0 && row_end <= e0 + cnt) {
+        float res[VEC];
+#pragma unroll
+        for (int c = 0; c < VEC; ++c)
+          res[c] = MEAN ? acc[c] / static_cast<float>(row_end - row_start) : acc[c];  // reducer.cuh:75-76
         store_vec<VEC>(dst, res);
       } else {
+        // a row cut by a chunk boundary: its partial SUMS meet in memory; for the mean,
+        // spmm_mean_finish_kernel divides the total once, as the reference's reducer does
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) unsafeAtomicAdd(dst + c, res[c]);
+        for (int c = 0; c < VEC; ++c) unsafeAtomicAdd(dst + c, acc[c]);
       }
     }
 #pragma unroll
@@ -168,7 +196,7 @@ __global__ __launch_bounds__(kBlock) void spmm_chunk_kernel(const I* __restrict_
       for (int c = 0; c < VEC; ++c) xv[u][c] = 0.f;
       if (base + u < cnt) {  // wave-uniform, so every lane takes part in the broadcast
         const int64_t c = readlane_i(my_col, base + u);
-        if (kok) load_vec<VEC>(X + c * K + kcol, xv[u]);
+        if (kok) load_vec<VEC>(X + c * ldx + kcol, xv[u]);
       }
     }
 #pragma unroll
@@ -192,7 +220,7 @@ static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>
 
 template <typename I, int VEC>
 static void spmm_dispatch(const I* rowptr, const I* col, const float* val, const float* X, int64_t M,
-                          int64_t nnz, int64_t K, int reduce, float* out, hipStream_t s) {
+                          int64_t nnz, int64_t K, int64_t ldx, int64_t ldo, int reduce, float* out, hipStream_t s) {
   const int64_t chunks = (nnz + kChunk - 1) / kChunk;
   const int64_t wgs = (chunks + 3) / 4;
   const dim3 grid(static_cast<unsigned>((wgs + kXcds - 1) / kXcds * kXcds),
@@ -200,11 +228,11 @@ static void spmm_dispatch(const I* rowptr, const I* col, const float* val, const
   const dim3 block(kBlock);
   const bool mean = reduce == EXACT_REDUCE_MEAN;
   if (val) {
-    if (mean) hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, true, true>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, out);
-    else hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, true, false>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, out);
+    if (mean) hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, true, true>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, ldx, ldo, out);
+    else hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, true, false>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, ldx, ldo, out);
   } else {
-    if (mean) hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, false, true>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, out);
-    else hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, false, false>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, out);
+    if (mean) hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, false, true>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, ldx, ldo, out);
+    else hipLaunchKernelGGL((spmm_chunk_kernel<I, VEC, false, false>), grid, block, 0, s, rowptr, col, val, X, M, nnz, K, ldx, ldo, out);
   }
 }
 
@@ -214,25 +242,26 @@ using namespace exact;
 
 extern "C" {
 
-int exact_spmm_csr_f32(const void* rowptr, const void* col, const float* val, int idx_bytes,
-                       const float* X, int64_t M, int64_t n_cols, int64_t K, int64_t nnz, int reduce,
-                       float* out, void* stream) {
+int exact_spmm_csr_strided_f32(const void* rowptr, const void* col, const float* val, int idx_bytes,
+                               const float* X, int64_t ldx, int64_t M, int64_t n_cols, int64_t K, int64_t nnz,
+                               int reduce, float* out, int64_t ldo, void* stream) {
   if (idx_bytes != 4 && idx_bytes != 8) return EXACT_E_ARG;
   if (reduce != EXACT_REDUCE_SUM && reduce != EXACT_REDUCE_MEAN) return EXACT_E_ARG;
   if (M < 0 || K < 0 || nnz < 0 || n_cols < 0 || n_cols > 0x7FFFFFFFll) return EXACT_E_SHAPE;
   if (idx_bytes == 4 && nnz > 0x7FFFFFFFll) return EXACT_E_SHAPE;
   // launch-grid limits: 2^31 - 1 workgroups of 256 rows (pre-pass) resp. 256 entries (main kernel)
   if (M > (int64_t{1} << 38) || nnz > (int64_t{1} << 38) || K > (int64_t{1} << 24)) return EXACT_E_SHAPE;
+  if (ldx < K || ldo < K) return EXACT_E_SHAPE;
   if (M == 0 || K == 0) return EXACT_OK;
   if (!rowptr || !out || (nnz > 0 && (!col || !X))) return EXACT_E_NULL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 zgrid(static_cast<unsigned>((M + kBlock - 1) / kBlock));
   if (idx_bytes == 4)
     hipLaunchKernelGGL((spmm_zero_rows_kernel<int32_t>), zgrid, dim3(kBlock), 0, s,
-                       static_cast<const int32_t*>(rowptr), M, K, out);
+                       static_cast<const int32_t*>(rowptr), M, K, ldo, out);
   else
     hipLaunchKernelGGL((spmm_zero_rows_kernel<int64_t>), zgrid, dim3(kBlock), 0, s,
-                       static_cast<const int64_t*>(rowptr), M, K, out);
+                       static_cast<const int64_t*>(rowptr), M, K, ldo, out);
   if (nnz > 0) {
     // Column tile of one wavefront = 64 * vec columns.  Measured on power-law
     // graphs of 170k to 2.4M rows: 8-byte gathers (128-column tiles) beat 16-byte
@@ -240,18 +269,32 @@ int exact_spmm_csr_f32(const void* rowptr, const void* col, const float* val, in
     // as many wavefronts share the same gathers -- so 16-byte gathers are not
     // used; rows of at most 64 columns take 4-byte gathers (one tile, more lanes
     // busy than with wider ones).
-    const int vec = (K > 64 && K % 2 == 0 && al(X, 8) && al(out, 8)) ? 2 : 1;
+    const int vec = (K > 64 && K % 2 == 0 && ldx % 2 == 0 && ldo % 2 == 0 && al(X, 8) && al(out, 8)) ? 2 : 1;
     if ((K + kWave * vec - 1) / (kWave * vec) > 65535) return EXACT_E_SHAPE;  // grid.y limit
 #define EXACT_SPMM_GO(I, V) \
-  spmm_dispatch<I, V>(static_cast<const I*>(rowptr), static_cast<const I*>(col), val, X, M, nnz, K, reduce, out, s)
+  spmm_dispatch<I, V>(static_cast<const I*>(rowptr), static_cast<const I*>(col), val, X, M, nnz, K, ldx, ldo, reduce, out, s)
     if (idx_bytes == 4) {
       if (vec == 2) EXACT_SPMM_GO(int32_t, 2); else EXACT_SPMM_GO(int32_t, 1);
     } else {
       if (vec == 2) EXACT_SPMM_GO(int64_t, 2); else EXACT_SPMM_GO(int64_t, 1);
     }
 #undef EXACT_SPMM_GO
+    if (reduce == EXACT_REDUCE_MEAN) {
+      if (idx_bytes == 4)
+        hipLaunchKernelGGL((spmm_mean_finish_kernel<int32_t>), zgrid, dim3(kBlock), 0, s,
+                           static_cast<const int32_t*>(rowptr), M, K, ldo, out);
+      else
+        hipLaunchKernelGGL((spmm_mean_finish_kernel<int64_t>), zgrid, dim3(kBlock), 0, s,
+                           static_cast<const int64_t*>(rowptr), M, K, ldo, out);
+    }
   }
   return launch_status();
+}
+
+int exact_spmm_csr_f32(const void* rowptr, const void* col, const float* val, int idx_bytes,
+                       const float* X, int64_t M, int64_t n_cols, int64_t K, int64_t nnz, int reduce,
+                       float* out, void* stream) {
+  return exact_spmm_csr_strided_f32(rowptr, col, val, idx_bytes, X, K, M, n_cols, K, nnz, reduce, out, K, stream);
 }
 
 }  // extern "C"

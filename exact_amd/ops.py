@@ -506,7 +506,7 @@ class qbn_relu_dropout(Function):
                 exponential_average_factor, eps, p, bits, scheme):
         kept = CompressedActivation.compress(input, scheme, project=False)
         rows = input.shape[0]
-        var, mean = torch.var_mean(input, dim=0, unbiased=False)
+        var, mean = ext_backward_func.batch_statistics(input)
         invstd = torch.rsqrt(var + eps)
         if running_mean is not None:                       # the bookkeeping of native_batch_norm
             running_mean.mul_(1 - exponential_average_factor).add_(mean, alpha=exponential_average_factor)

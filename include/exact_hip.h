@@ -133,6 +133,14 @@ int exact_spmm_csr_f32(const void *rowptr, const void *col, const float *val,
                        int idx_bytes, const float *X, int64_t M, int64_t n_cols,
                        int64_t K, int64_t nnz, int reduce, float *out, void *stream);
 
+/* The same with explicit row strides (in elements, >= K) of X and out, for
+ * operands that are column slices of wider buffers -- e.g. rows padded to a
+ * multiple of 128 bytes, which the 512-byte gathers of the kernel like. */
+int exact_spmm_csr_strided_f32(const void *rowptr, const void *col, const float *val,
+                               int idx_bytes, const float *X, int64_t ldx, int64_t M,
+                               int64_t n_cols, int64_t K, int64_t nnz, int reduce,
+                               float *out, int64_t ldo, void *stream);
+
 /* The same product with a reproducible result: one wavefront per row, entries
  * added in CSR order with one multiply and one add each (the order of the
  * reference kernel, spmm_cuda.cu:85-90), no atomics.  Slower on hub rows. */
@@ -176,12 +184,30 @@ int exact_elu_bwd_f32(const float *dy, const float *x, float alpha, int64_t n,
 int exact_elu_bwd_f16(const uint16_t *dy, const uint16_t *x, float alpha, int64_t n,
                       uint16_t *dx, void *stream);
 
-/* Column sums of a row-major [N, K] fp32 matrix, out[k] = sum_n x[n, k], K <= 8192,
- * x 16-byte aligned.  Replaces `grad_output.sum(0)`, the bias gradient of
+/* Column sums of a row-major [N, K] fp32 matrix, out[k] = sum_n x[n, k], K <= 8192.  Replaces `grad_output.sum(0)`, the bias gradient of
  * linear_backward (backward_func.cc:90-91), whose library reduction is far off
  * the memory roofline for narrow matrices.  fp32 atomics: the summation order
  * is not fixed. */
 int exact_colsum_f32(const float *x, int64_t N, int64_t K, float *out, void *stream);
+
+/* The two column reductions of a training-mode batch norm's backward over
+ * row-major [N, K] fp32 matrices, K <= 256, in one pass:
+ *   sum_dy[k] = sum_n dy[n, k],  sum_dy_xmu[k] = sum_n dy[n, k] * (x[n, k] - mean[k]).
+ * Replaces the reduction inside at::native_batch_norm_backward as called by
+ * qbatch_norm.backward (ops.py:228-254); the element-wise half of that routine
+ * stays the framework's.  fp32 atomics: the summation order is not fixed. */
+int exact_bn_backward_reduce_f32(const float *dy, const float *x, const float *mean, int64_t N, int64_t K,
+                                 float *sum_dy, float *sum_dy_xmu, void *stream);
+
+/* Centred column moments of a row-major [N, K] fp32 matrix, K <= 256, in one pass:
+ *   sum_d[k] = sum_n (x[n, k] - center[k]),  sum_d2[k] = sum_n (x[n, k] - center[k])^2,
+ * from which mean = center + sum_d / N and the biased variance = sum_d2 / N - (sum_d / N)^2
+ * (free of cancellation when `center` is near the column means, e.g. the mean of a few rows).
+ * Replaces the batch statistics inside at::native_batch_norm as called by
+ * qbatch_norm.forward (ops.py:213) where the normalisation itself is folded
+ * into the next pass.  fp32 atomics: the summation order is not fixed. */
+int exact_col_moments_f32(const float *x, const float *center, int64_t N, int64_t K, float *sum_d, float *sum_d2,
+                          void *stream);
 
 /* Fused epilogues (no single counterpart in the reference: each replaces a
  * chain of its calls with one pass over the data, bit-identical to the chain).

@@ -432,6 +432,26 @@ static void check_colsum(int64_t N, int64_t K, std::mt19937& rng) {
   CHECK(rc == 0, "colsum rc %d N=%lld K=%lld", rc, (long long)N, (long long)K);
   for (int64_t k = 0; k < K; ++k)
     CHECK(out[k] == static_cast<float>(want[static_cast<size_t>(k)]), "colsum N=%lld K=%lld col %lld", (long long)N, (long long)K, (long long)k);
+  if (K > 256) return;
+  // the two-matrix and the centred-moment forms of the same kernel (small integers: exact)
+  Buf<float> y(static_cast<size_t>(N * K)), ctr(static_cast<size_t>(K)), a(static_cast<size_t>(K)), b(static_cast<size_t>(K));
+  for (int64_t k = 0; k < K; ++k) ctr[k] = static_cast<float>(id(rng) / 4);
+  for (int64_t i = 0; i < N * K; ++i) y[i] = static_cast<float>(id(rng) / 2);
+  std::vector<double> w1(static_cast<size_t>(K), 0.0), w2(static_cast<size_t>(K), 0.0), m1(static_cast<size_t>(K), 0.0);
+  for (int64_t i = 0; i < N * K; ++i) {
+    const size_t k = static_cast<size_t>(i % K);
+    w1[k] += x[i] * (y[i] - ctr[k]);
+    m1[k] += (x[i] - ctr[k]);
+    w2[k] += (x[i] - ctr[k]) * (x[i] - ctr[k]);
+  }
+  CHECK(exact_bn_backward_reduce_f32(x.p, y.p, ctr.p, N, K, a.p, b.p, nullptr) == 0, "bn reduce rc");
+  for (int64_t k = 0; k < K; ++k)
+    CHECK(a[k] == static_cast<float>(want[static_cast<size_t>(k)]) && b[k] == static_cast<float>(w1[static_cast<size_t>(k)]),
+          "bn reduce N=%lld K=%lld col %lld", (long long)N, (long long)K, (long long)k);
+  CHECK(exact_col_moments_f32(x.p, ctr.p, N, K, a.p, b.p, nullptr) == 0, "moments rc");
+  for (int64_t k = 0; k < K; ++k)
+    CHECK(a[k] == static_cast<float>(m1[static_cast<size_t>(k)]) && b[k] == static_cast<float>(w2[static_cast<size_t>(k)]),
+          "moments N=%lld K=%lld col %lld", (long long)N, (long long)K, (long long)k);
 }
 
 int main(int argc, char** argv) {

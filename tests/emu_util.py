@@ -383,3 +383,31 @@ def colsum(x, guard=8, expect_rc=0):
         return None
     assert (out[K:] == np.float32(-777.0)).all()
     return out[:K]
+
+
+def bn_backward_reduce(dy, x, mean, guard=8, expect_rc=0):
+    """exact_bn_backward_reduce_f32 -> (sum_dy, sum_dy_xmu), fp32 [K] each."""
+    dy, x, mean = f32(dy), f32(x), f32(mean)
+    N, K = dy.shape
+    a = np.full(K + guard, np.float32(-777.0), np.float32)
+    b = np.full(K + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_bn_backward_reduce_f32(p(dy), p(x), p(mean), N, K, p(a), p(b), None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (a[K:] == np.float32(-777.0)).all() and (b[K:] == np.float32(-777.0)).all()
+    return a[:K], b[:K]
+
+
+def col_moments(x, center, guard=8, expect_rc=0):
+    """exact_col_moments_f32 -> (sum of (x - center), sum of (x - center)^2), fp32 [K] each."""
+    x, center = f32(x), f32(center)
+    N, K = x.shape
+    a = np.full(K + guard, np.float32(-777.0), np.float32)
+    b = np.full(K + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_col_moments_f32(p(x), p(center), N, K, p(a), p(b), None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (a[K:] == np.float32(-777.0)).all() and (b[K:] == np.float32(-777.0)).all()
+    return a[:K], b[:K]

@@ -563,3 +563,112 @@ def test_bias_gradient_goes_through_the_column_sum_kernel(backend):
         assert torch.equal(bf.column_sums(ints), ints.sum(0))
     small = torch.randn(10, 3).to(backend)
     assert torch.equal(bf.column_sums(small), small.sum(0))       # short matrices keep the framework's reduction
+
+
+@pytest.mark.parametrize("N,K", [(1, 1), (3, 5), (7, 47), (1000, 40), (4099, 64), (513, 256), (2050, 100), (40000, 3)])
+def test_batch_norm_backward_reduction_kernel(N, K):
+    """exact_bn_backward_reduce_f32: sum of dy and of dy * (x - mean) per column.
+    Small integers make every product and sum exact, so a misplaced or repeated
+    element shows; random data within fp32 summation error of float64."""
+    rng = np.random.default_rng(N + 13 * K)
+    dy = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    x = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    mean = rng.integers(-2, 3, K).astype(np.float32)
+    a, b = e.bn_backward_reduce(dy, x, mean)
+    assert np.array_equal(a, dy.astype(np.float64).sum(0).astype(np.float32))
+    assert np.array_equal(b, (dy.astype(np.float64) * (x - mean)).sum(0).astype(np.float32))
+    dy, x = rng.standard_normal((N, K)).astype(np.float32), rng.standard_normal((N, K)).astype(np.float32) * 2 + 1
+    mean = x.mean(0)
+    a, b = e.bn_backward_reduce(dy, x, mean)
+    prod = dy.astype(np.float64) * (x.astype(np.float64) - mean)
+    assert np.allclose(a, dy.astype(np.float64).sum(0), rtol=0, atol=1e-6 * np.abs(dy).astype(np.float64).sum(0).max())
+    assert np.allclose(b, prod.sum(0), rtol=0, atol=2e-6 * np.abs(prod).sum(0).max())
+    assert e.bn_backward_reduce(np.zeros((2, 257), np.float32), np.zeros((2, 257), np.float32), np.zeros(257, np.float32),
+                                expect_rc=-3) is None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,K,affine", [(169343, 256, True), (5000, 64, True), (20000, 40, False), (4097, 100, True)])
+def test_batch_norm_backward_with_the_one_pass_reduction(cuda, N, K, affine):
+    """native_batch_norm_backward through the library's column reduction + the
+    framework's element-wise half, against the framework's one-call routine
+    (what qbatch_norm.backward calls, ops.py:228-254)."""
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator(device=cuda).manual_seed(N + K)
+    x = torch.randn(N, K, generator=g, device=cuda) * 1.5 + 0.3
+    dy = torch.randn(N, K, generator=g, device=cuda)
+    w = torch.rand(K, generator=g, device=cuda) + 0.5 if affine else None
+    var, mean = torch.var_mean(x, dim=0, unbiased=False)
+    invstd = torch.rsqrt(var + 1e-5)
+    for mask in ([True, True, True], [True, False, False], [False, True, True]):
+        mask = [mask[0], mask[1] and affine, mask[2] and affine]
+        want = torch.ops.aten.native_batch_norm_backward(dy, x, w, None, None, mean, invstd, True, 1e-5, mask)
+        got = bf.native_batch_norm_backward(dy, x, w, None, None, mean, invstd, True, 1e-5, mask)
+        for a, b, m in zip(got, want, mask):
+            if not m:
+                assert a is None
+                continue
+            scale = b.abs().max().item() + 1e-12
+            assert (a - b).abs().max().item() <= 2e-5 * scale, (mask, (a - b).abs().max().item(), scale)
+
+
+@pytest.mark.parametrize("N,K", [(1, 1), (3, 5), (7, 47), (1000, 40), (4099, 64), (513, 256), (2050, 100)])
+def test_column_moments_kernel(N, K):
+    """exact_col_moments_f32: exact on small integers; on data with a mean far
+    from zero the variance formed from the centred moments keeps its digits."""
+    rng = np.random.default_rng(N + 17 * K)
+    x = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    c = x[0].copy()
+    a, b = e.col_moments(x, c)
+    d = x.astype(np.float64) - c
+    assert np.array_equal(a, d.sum(0).astype(np.float32)) and np.array_equal(b, (d * d).sum(0).astype(np.float32))
+    x = (rng.standard_normal((N, K)) * 0.5 + 100.0).astype(np.float32)      # mean 200 standard deviations from zero
+    a, b = e.col_moments(x, x[0])
+    shift = a.astype(np.float64) / N
+    var = b.astype(np.float64) / N - shift * shift
+    want = x.astype(np.float64).var(0)
+    assert np.allclose(x[0] + shift, x.astype(np.float64).mean(0), rtol=1e-6)
+    if N > 100:
+        assert np.allclose(var, want, rtol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,K", [(169343, 256), (5000, 64), (20000, 40)])
+def test_batch_statistics_match_var_mean(cuda, N, K):
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator(device=cuda).manual_seed(N)
+    x = torch.randn(N, K, generator=g, device=cuda) * 1.5 + 3.0
+    var, mean = bf.batch_statistics(x)
+    want_var, want_mean = torch.var_mean(x.double(), dim=0, unbiased=False)
+    assert (mean.double() - want_mean).abs().max().item() < 1e-5
+    assert ((var.double() - want_var) / want_var).abs().max().item() < 1e-5
+
+
+def test_sparse_product_with_row_strides(backend):
+    """The dense operand as a column slice of a wider buffer (unit column
+    stride, longer row stride) and the padded copy the shim makes of wide,
+    unaligned rows on dense graphs: same product, nothing outside the slice is
+    read into the result."""
+    import scipy.sparse as sp
+    from exact_amd.cpp_extension import spmm as ext_spmm
+    rng = np.random.default_rng(3)
+    n, K = 300, 130                                          # 130 columns: > 128 and not a multiple of 32
+    A = sp.random(n, n, density=0.08, format="csr", random_state=4, dtype=np.float32)   # ~24 entries per row >= 16
+    A.sort_indices()
+    rowptr = torch.from_numpy(A.indptr.astype(np.int64)).to(backend)
+    col = torch.from_numpy(A.indices.astype(np.int64)).to(backend)
+    val = torch.from_numpy(A.data).to(backend)
+    X = rng.standard_normal((n, K)).astype(np.float32)
+    wide = torch.full((n, K + 37), float("nan"))
+    wide[:, 5:5 + K] = torch.from_numpy(X)
+    wide = wide.to(backend)
+    for reduce in ("sum", "mean"):
+        want = o.spmm_csr(A.indptr, A.indices, A.data, X, reduce)
+        scale = np.abs(want).max()
+        got_view = ext_spmm.spmm_csr(rowptr, col, val, wide[:, 5:5 + K], reduce)          # strided, no copy
+        got_pad = ext_spmm.spmm_csr(rowptr, col, val, torch.from_numpy(X).to(backend), reduce)   # padded copy
+        assert np.allclose(got_view.cpu().numpy(), want, rtol=0, atol=1e-5 * scale)
+        assert np.allclose(got_pad.cpu().numpy(), want, rtol=0, atol=1e-5 * scale)
+    padded = ext_spmm._aligned_rows(torch.from_numpy(X).to(backend), A.nnz)
+    assert padded.shape == (n, K) and padded.stride(0) == 160 and padded.stride(1) == 1
+    assert ext_spmm._aligned_rows(wide[:, 5:5 + K], A.nnz).data_ptr() == wide[:, 5:5 + K].data_ptr()
