@@ -380,6 +380,9 @@ def _profile_target(argv=None):
     ap.add_argument("--cols", type=int, default=256)
     ap.add_argument("--reps", type=int, default=100)
     ap.add_argument("--supplied-noise", action="store_true")
+    ap.add_argument("--config", choices=sorted(EPOCH_CONFIGS), default="cfg3_gcn_int2",
+                    help="spmm only: the graph of this model configuration")
+    ap.add_argument("--width", type=int, default=0, help="spmm only: columns of the dense operand (0 = --cols)")
     args = ap.parse_args(argv)
     dev = bench_device()
     L = _lib.lib()
@@ -401,8 +404,12 @@ def _profile_target(argv=None):
     packed_k = torch.empty(int(L.exact_packed_nbytes(N, k, b)), dtype=torch.int8, device=dev)
     ones = torch.ones(G, device=dev)
     if args.kernel == "spmm":
-        adj = gcn_norm(powerlaw_graph(N, int(N * 6.85), seed=1, device=dev)).to_int32_()
+        kind, n_nodes, n_edges = EPOCH_CONFIGS[args.config][:3]
+        adj = powerlaw_graph(n_nodes, n_edges, seed=1, device=dev)
+        adj = (gcn_norm(adj) if kind == "gcn" else adj).to_int32_()
         rowptr, col, value = adj.csr()
+        spmm_x = torch.randn((n_nodes, args.width or G), generator=gen, device=dev)
+        spmm_reduce = "sum" if kind == "gcn" else "mean"
     fns = {
         "pack": lambda i: L.exact_minmax_pack_f32(x.data_ptr(), noise.data_ptr() if noise is not None else None, 1,
                                                   i, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),
@@ -423,7 +430,7 @@ def _profile_target(argv=None):
                                                         sp),
         "rp_fwd": lambda i: L.exact_rp_fwd_f32(x.data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp),
         "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, out.data_ptr(), sp),
-        "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, x, "sum"),
+        "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, spmm_x, spmm_reduce),
         "copy": lambda i: out.copy_(x),
     }
     fn = fns[args.kernel]

@@ -48,11 +48,34 @@ def batch_statistics(matrix):
     return (sums[1] / N - shift * shift).clamp_(min=0.0), center + shift
 
 
+def weight_gradient(grad_output, input):  # noqa: A002
+    """`grad_output.t().mm(input)` (backward_func.cc:88-89): [N, out]^T . [N, in].
+    Tall fp32 device operands take the library's matrix-core kernel for this
+    shape (its slabs meet through atomics, so deterministic mode and everything
+    else keep the framework's GEMM)."""
+    usable = (grad_output.dim() == 2 and input.dim() == 2 and grad_output.dtype == torch.float32
+              and input.dtype == torch.float32 and _checks.on_device(grad_output) and _checks.on_device(input)
+              and grad_output.shape[0] == input.shape[0] and grad_output.shape[0] >= 16384
+              and 0 < grad_output.shape[1] <= 1024 and 0 < input.shape[1] <= 1024
+              and grad_output.stride(1) == 1 and input.stride(1) == 1
+              and grad_output.stride(0) >= grad_output.shape[1] and input.stride(0) >= input.shape[1]
+              and not torch.are_deterministic_algorithms_enabled())
+    if not usable:
+        return grad_output.t().mm(input)
+    N, K = grad_output.shape
+    D = input.shape[1]
+    out = torch.empty((K, D), dtype=torch.float32, device=grad_output.device)
+    rc = _lib.lib().exact_linear_dw_f32(_checks.ptr(grad_output), grad_output.stride(0), _checks.ptr(input), input.stride(0),
+                                        N, K, D, _checks.ptr(out), _checks.stream_ptr(grad_output))
+    _lib.check(rc, "weight_gradient")
+    return out
+
+
 def linear_backward(grad_output, input, weight, bias, need_input_grad=True):  # noqa: A002
     """backward_func.cc:83-93.  `need_input_grad=False` leaves out the product
     the caller would discard (the reference forms all three regardless)."""
     grad_input = grad_output.mm(weight) if need_input_grad else None
-    grad_weight = grad_output.t().mm(input)
+    grad_weight = weight_gradient(grad_output, input)
     grad_bias = column_sums(grad_output) if bias is not None else None
     return grad_input, grad_weight, grad_bias
 

@@ -4,9 +4,9 @@ argument lists, plus spmm_value_bw (the edge-value gradient).
 """
 from __future__ import annotations
 
-from collections import OrderedDict
 
 import torch
+from torch.utils.weak import WeakIdKeyDictionary
 
 from .. import _lib
 from ..conf import config
@@ -124,33 +124,35 @@ def spmm_mean_fw(row, rowptr, col, value, rowcount, colptr, csr2csc, mat):
 
 # The reference re-gathers row[csr2csc], value[csr2csc] (and the mean weights)
 # with index_select on EVERY backward (spmm.cc:73-75, 129-133).  They depend
-# only on the graph, so they are built once per (graph, values) and kept.
-_CSC_CACHE: "OrderedDict[tuple, tuple]" = OrderedDict()
-_CSC_CACHE_MAX = 16
+# only on the graph, so they are built once and kept -- attached to the graph's
+# own `csr2csc` tensor (the object a SparseTensor's storage caches), weakly: the
+# entry dies with the graph, and a graph rebuilt every step (gcn_norm without
+# caching, learned or attention edge values) leaves nothing behind.  Per graph
+# there is ONE slot per reduction for the value-dependent part, replaced when
+# the values change; values that require grad change every step and are never
+# kept.
+_CSC_CACHE = WeakIdKeyDictionary()          # csr2csc tensor -> {"row_csc": .., "sum": (tag, w), "mean": (tag, w)}
 
 
 def _csc_operands(kind, row, value, rowcount, csr2csc, has_value, dtype):
-    key = (kind, row.data_ptr(), csr2csc.data_ptr(), row.numel(),
-           value.data_ptr() if has_value else 0, value._version if has_value else 0,
-           rowcount.data_ptr() if rowcount is not None else 0)
-    # fp16 values are per-call copies made by autocast: nothing to reuse, nothing to keep
-    cacheable = not (has_value and value.dtype != torch.float32)
-    hit = _CSC_CACHE.get(key) if cacheable else None
-    if hit is not None:
-        _CSC_CACHE.move_to_end(key)
-        return hit[0], hit[1]
-    row_csc = row.index_select(0, csr2csc)
+    # fp16 values are per-call copies made by autocast, values that require grad are new every step
+    cacheable = not (has_value and (value.dtype != torch.float32 or value.requires_grad))
+    slot = _CSC_CACHE.get(csr2csc) if cacheable else None
+    if slot is not None and slot["row"] != (row.data_ptr(), row.numel()):
+        slot = None                                         # the same permutation handed in with other rows
+    tag = (value.data_ptr(), value._version) if has_value else None
+    if slot is not None and kind in slot and slot[kind][0] == tag:
+        return slot["row_csc"], slot[kind][1]
+    row_csc = slot["row_csc"] if slot is not None else row.index_select(0, csr2csc)
     if kind == "sum":
         w = value.detach().index_select(0, csr2csc) if has_value else None
     else:
         cnt = rowcount.to(torch.float32).index_select(0, row_csc).clamp_(min=1)   # fp32 whatever `dtype` is
         w = value.detach().index_select(0, csr2csc).div(cnt) if has_value else cnt.pow_(-1)
-    if not cacheable:
-        return row_csc, w
-    # the inputs are kept alive with the entry so their addresses cannot be reused
-    _CSC_CACHE[key] = (row_csc, w, (row, value, rowcount, csr2csc))
-    while len(_CSC_CACHE) > _CSC_CACHE_MAX:
-        _CSC_CACHE.popitem(last=False)
+    if cacheable:
+        if slot is None:
+            slot = _CSC_CACHE[csr2csc] = {"row": (row.data_ptr(), row.numel()), "row_csc": row_csc, "keep": row}
+        slot[kind] = (tag, w)
     return row_csc, w
 
 

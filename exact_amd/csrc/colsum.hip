@@ -155,6 +155,16 @@ __global__ __launch_bounds__(kBlock) void colsum_wide_kernel(const float* __rest
 
 using namespace exact;
 
+// Every workgroup ends with one atomic add per column into the SAME K words,
+// and atomics on one address are served one after the other: a few hundred
+// long-lived workgroups (about 1024, at least 16 KiB of the stream each)
+// instead of thousands of short ones.
+static int64_t colsum_rows_per_wg(int64_t N, int64_t K) {
+  int64_t rows = (N + 1023) / 1024;
+  const int64_t least = (4096 + K - 1) / K;
+  return rows < least ? least : rows;
+}
+
 extern "C" {
 
 int exact_colsum_f32(const float* x, int64_t N, int64_t K, float* out, void* stream) {
@@ -164,9 +174,7 @@ int exact_colsum_f32(const float* x, int64_t N, int64_t K, float* out, void* str
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(colsum_zero_kernel, dim3(static_cast<unsigned>((K + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, out, K);
   if (N > 0) {
-    // about 64 KiB of the stream per workgroup, at most 8192 workgroups
-    int64_t rows_per_wg = (16384 + K - 1) / K;
-    if ((N + rows_per_wg - 1) / rows_per_wg > 8192) rows_per_wg = (N + 8191) / 8192;
+    int64_t rows_per_wg = colsum_rows_per_wg(N, K);
     const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg));
     if (K <= kBlock) {
       const bool vec4 = (K % 4 == 0) && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
@@ -196,8 +204,7 @@ int exact_bn_backward_reduce_f32(const float* dy, const float* x, const float* m
   if (N > 0) {
     const bool vec4 = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0;
     const int rpp = static_cast<int>(kBlock / (vec4 ? K / 4 : K));
-    int64_t rows_per_wg = (8192 + K - 1) / K;  // about 32 KiB of each matrix per workgroup
-    if ((N + rows_per_wg - 1) / rows_per_wg > 8192) rows_per_wg = (N + 8191) / 8192;
+    int64_t rows_per_wg = colsum_rows_per_wg(N, K);
     rows_per_wg = (rows_per_wg + rpp - 1) / rpp * rpp;  // whole passes
     const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg));
     if (vec4) hipLaunchKernelGGL((colsum_narrow_kernel<4, true>), grid, dim3(kBlock), 0, s, dy, x, mean, N, static_cast<int>(K), rpp, rows_per_wg, sum_dy, sum_dy_xmu);
@@ -218,8 +225,7 @@ int exact_col_moments_f32(const float* x, const float* center, int64_t N, int64_
   if (N > 0) {
     const bool vec4 = (K % 4 == 0) && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     const int rpp = static_cast<int>(kBlock / (vec4 ? K / 4 : K));
-    int64_t rows_per_wg = (16384 + K - 1) / K;
-    if ((N + rows_per_wg - 1) / rows_per_wg > 8192) rows_per_wg = (N + 8191) / 8192;
+    int64_t rows_per_wg = colsum_rows_per_wg(N, K);
     rows_per_wg = (rows_per_wg + rpp - 1) / rpp * rpp;  // whole passes
     const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg));
     const float* none = nullptr;

@@ -25,6 +25,13 @@ namespace exact {
 constexpr int kChunk = 64;  // entries per wavefront == lanes per wavefront
 constexpr int kGather = 8;  // X rows in flight per lane (4 and 16 measure the same)
 constexpr int kXcds = 8;    // accelerator complex dies of an MI355X, each with its own L2
+// Mean aggregation, rows cut by chunk boundaries: up to this length every chunk
+// divides its partial sum by the row length before the atomic add (at most 32
+// rounded terms); longer rows -- the hubs -- add raw partial sums and are
+// divided once by spmm_mean_finish_kernel, like the reference's reducer, so
+// hundreds of rounded quotients never pile up.  Dividing every split row at
+// the end would re-read and re-write most of the output on dense graphs.
+constexpr int64_t kMeanFinishLen = 2048;
 
 template <int VEC> struct Vec;
 template <> struct Vec<2> { using T = float2; };
@@ -75,8 +82,9 @@ __global__ __launch_bounds__(kBlock) void spmm_zero_rows_kernel(const I* __restr
   }
 }
 
-// Mean aggregation, rows that span more than one chunk: the chunk kernel has
-// added up their partial sums; divide by the row length (reducer.cuh:75-76).
+// Mean aggregation, rows longer than kMeanFinishLen that span more than one
+// chunk: the chunk kernel has added up their partial sums; divide by the row
+// length (reducer.cuh:75-76).
 template <typename I>
 __global__ __launch_bounds__(kBlock) void spmm_mean_finish_kernel(const I* __restrict__ rowptr, int64_t M,
                                                                   int64_t K, int64_t ldo, float* __restrict__ out) {
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(kBlock) void spmm_mean_finish_kernel(const I* __res
   float len = 1.f;
   if (r < M) {
     const int64_t rs = rowptr[r], re = rowptr[r + 1];
-    split = (re > rs) && (rs / kChunk != (re - 1) / kChunk);
+    split = (re - rs > kMeanFinishLen) && (rs / kChunk != (re - 1) / kChunk);
     len = static_cast<float>(re - rs);
   }
   uint64_t todo = __ballot(split);
@@ -168,10 +176,11 @@ __global__ __launch_bounds__(kBlock) void spmm_chunk_kernel(const I* __restrict_
           res[c] = MEAN ? acc[c] / static_cast<float>(row_end - row_start) : acc[c];  // reducer.cuh:75-76
         store_vec<VEC>(dst, res);
       } else {
-        // a row cut by a chunk boundary: its partial SUMS meet in memory; for the mean,
-        // spmm_mean_finish_kernel divides the total once, as the reference's reducer does
+        // a row cut by a chunk boundary: its partial sums meet in memory
+        const int64_t len = row_end - row_start;
+        const float div = (MEAN && len <= kMeanFinishLen) ? static_cast<float>(len) : 1.f;
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) unsafeAtomicAdd(dst + c, acc[c]);
+        for (int c = 0; c < VEC; ++c) unsafeAtomicAdd(dst + c, MEAN ? acc[c] / div : acc[c]);
       }
     }
 #pragma unroll

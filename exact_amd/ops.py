@@ -276,7 +276,7 @@ class qlinear(Function):
             # which fp32 sums are taken differs.
             x_r = dequantize_activation(kept.quantized, kept.stored_shape)
             grad_input = grad_output.mm(ctx.weight) if ctx.needs_input_grad[0] else None
-            grad_weight = grad_output.t().mm(x_r).mm(kept.randmat.t())
+            grad_weight = ext_backward_func.weight_gradient(grad_output, x_r).mm(kept.randmat.t())
             grads = (grad_input, grad_weight,
                      ext_backward_func.column_sums(grad_output) if ctx.bias is not None else None)
         empty_cache(config.empty_cache_threshold)

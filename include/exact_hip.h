@@ -209,6 +209,14 @@ int exact_bn_backward_reduce_f32(const float *dy, const float *x, const float *m
 int exact_col_moments_f32(const float *x, const float *center, int64_t N, int64_t K, float *sum_d, float *sum_d2,
                           void *stream);
 
+/* Weight gradient of a linear layer, dW[Kout, D] = dY[N, Kout]^T . X[N, D], row-major
+ * fp32 with row strides ldy >= Kout and ldx >= D (in elements), N >> Kout, D.
+ * Replaces `grad_output.t().mm(input)` of linear_backward (backward_func.cc:88-89)
+ * with an fp32 matrix-core kernel shaped for the long reduction.  The row range
+ * is cut into slabs combined by fp32 atomics: the summation order is not fixed. */
+int exact_linear_dw_f32(const float *dY, int64_t ldy, const float *X, int64_t ldx, int64_t N,
+                        int64_t Kout, int64_t D, float *out, void *stream);
+
 /* Fused epilogues (no single counterpart in the reference: each replaces a
  * chain of its calls with one pass over the data, bit-identical to the chain).
  *

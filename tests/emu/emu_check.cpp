@@ -454,6 +454,23 @@ static void check_colsum(int64_t N, int64_t K, std::mt19937& rng) {
           "moments N=%lld K=%lld col %lld", (long long)N, (long long)K, (long long)k);
 }
 
+static void check_dw(int64_t N, int64_t K, int64_t D, int64_t pad, std::mt19937& rng) {
+  std::uniform_int_distribution<int> id(-3, 3);
+  const int64_t ldy = K + pad, ldx = D + 2 * pad;
+  Buf<float> dy(static_cast<size_t>(N * ldy)), x(static_cast<size_t>(N * ldx)), out(static_cast<size_t>(K * D));
+  for (int64_t i = 0; i < N * ldy; ++i) dy[i] = static_cast<float>(id(rng));
+  for (int64_t i = 0; i < N * ldx; ++i) x[i] = static_cast<float>(id(rng));
+  const int rc = exact_linear_dw_f32(dy.p, ldy, x.p, ldx, N, K, D, out.p, nullptr);
+  CHECK(rc == 0, "dw rc %d", rc);
+  for (int64_t k = 0; k < K; ++k)
+    for (int64_t d = 0; d < D; ++d) {
+      double want = 0;
+      for (int64_t n = 0; n < N; ++n) want += static_cast<double>(dy[n * ldy + k]) * x[n * ldx + d];
+      CHECK(out[k * D + d] == static_cast<float>(want), "dw N=%lld K=%lld D=%lld at (%lld, %lld)", (long long)N,
+            (long long)K, (long long)D, (long long)k, (long long)d);
+    }
+}
+
 int main(int argc, char** argv) {
   std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
@@ -500,6 +517,10 @@ int main(int argc, char** argv) {
   const int64_t cs[][2] = {{1, 1}, {3, 5}, {7, 47}, {1000, 41}, {4099, 47}, {513, 256}, {33, 602}, {5, 8192}, {20000, 3}};
   for (auto& c : cs) check_colsum(c[0], c[1], rng);
   std::printf("column sums ok (failures so far %d)\n", g_fail);
+  const int64_t ds[][4] = {{1, 1, 1, 0}, {7, 3, 5, 1}, {100, 40, 256, 0}, {515, 256, 128, 3}, {333, 47, 25, 0}, {1201, 256, 76, 2},
+                           {600, 130, 70, 0}, {513, 32, 200, 5}};
+  for (auto& d : ds) check_dw(d[0], d[1], d[2], d[3], rng);
+  std::printf("weight gradient ok (failures so far %d)\n", g_fail);
   if (mode == "large" || mode == "full") {
     for (int bits : {1, 2, 4, 8}) check_quant(20011, 256, bits, bits == 4, rng);
     check_quant(3001, 1024, 2, false, rng);

@@ -411,3 +411,21 @@ def col_moments(x, center, guard=8, expect_rc=0):
         return None
     assert (a[K:] == np.float32(-777.0)).all() and (b[K:] == np.float32(-777.0)).all()
     return a[:K], b[:K]
+
+
+def linear_dw(dy, x, ldy=None, ldx=None, guard=8, expect_rc=0):
+    """exact_linear_dw_f32 -> fp32 [Kout, D]; dy / x may be given wider than used (row strides)."""
+    dy, x = f32(dy), f32(x)
+    N, K = dy.shape
+    D = x.shape[1]
+    if ldy:
+        wide = np.full((N, ldy), np.float32(np.nan), np.float32); wide[:, :K] = dy; dy = wide
+    if ldx:
+        wide = np.full((N, ldx), np.float32(np.nan), np.float32); wide[:, :D] = x; x = wide
+    out = np.full(K * D + guard, np.float32(-777.0), np.float32)
+    rc = emu().exact_linear_dw_f32(p(dy), dy.shape[1], p(x), x.shape[1], N, K, D, p(out), None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (out[K * D:] == np.float32(-777.0)).all()
+    return out[:K * D].reshape(K, D)

@@ -120,6 +120,20 @@ def test_spmm_all_empty_and_single_long_row():
     col = np.random.default_rng(0).integers(0, 5, 1003)
     got = e.spmm(rowptr, col, None, X, "sum")
     assert np.array_equal(got[:, 0], np.array([0, 1000, 0, 3], F32))
+    # mean over a hub row (longer than the 2048 entries up to which every chunk divides its own partial sum:
+    # its raw partial sums are added up and divided once), next to a split row below that length
+    rng = np.random.default_rng(1)
+    rowptr = np.array([0, 7, 2600, 2600, 2900, 2903], np.int64)
+    col = rng.integers(0, 40, 2903)
+    val = rng.standard_normal(2903).astype(F32)
+    X = rng.standard_normal((40, 72)).astype(F32)
+    for v in (None, val):
+        want = o.spmm_csr(rowptr, col, v, X, "mean")
+        got = e.spmm(rowptr, col, v, X, "mean")
+        np.testing.assert_allclose(got, want, rtol=0, atol=1e-5 * np.abs(want).max())
+    ones = e.spmm(rowptr, col, None, np.ones((40, 8), F32), "mean")
+    assert np.array_equal(ones[1], np.ones(8, F32)) and np.array_equal(ones[2], np.zeros(8, F32))
+    np.testing.assert_allclose(ones[[0, 3, 4]], 1.0, rtol=0, atol=1e-6)
 
 
 @pytest.mark.parametrize("dist", ["rademacher", "gaussian"])

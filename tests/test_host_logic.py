@@ -118,3 +118,46 @@ def test_helpers():
     assert ops.kept_columns(256) == 32 and ops.kept_columns(602) == 76
     config.kept_frac = 0.25
     assert ops.kept_columns(100) == 25
+
+
+def test_transpose_operands_are_kept_per_graph_and_die_with_it():
+    """The gathered CSC operands of backward are attached to the graph's own
+    csr2csc tensor: a second call reuses them, new edge values replace the one
+    slot, values that require grad are never kept, and a graph that goes away
+    leaves nothing behind."""
+    import gc
+
+    import torch
+
+    from exact_amd.cpp_extension import spmm as ext_spmm
+    ext_spmm.clear_csc_cache()
+
+    def graph(seed):
+        g = torch.Generator().manual_seed(seed)
+        row = torch.sort(torch.randint(0, 50, (400,), generator=g)).values
+        csr2csc = torch.randperm(400, generator=g)
+        rowcount = torch.bincount(row, minlength=50)
+        return row, csr2csc, rowcount, torch.rand(400, generator=g)
+
+    row, csr2csc, rowcount, value = graph(0)
+    a = ext_spmm._csc_operands("sum", row, value, None, csr2csc, True, torch.float32)
+    b = ext_spmm._csc_operands("sum", row, value, None, csr2csc, True, torch.float32)
+    assert a[0] is b[0] and a[1] is b[1] and torch.equal(a[1], value[csr2csc]) and torch.equal(a[0], row[csr2csc])
+    m = ext_spmm._csc_operands("mean", row, None, rowcount, csr2csc, False, torch.float32)
+    assert m[0] is a[0] and torch.equal(m[1], 1.0 / rowcount[row[csr2csc]].clamp(min=1).float())
+    value.mul_(2.0)                                           # same storage, new version: the slot is rebuilt
+    c = ext_spmm._csc_operands("sum", row, value, None, csr2csc, True, torch.float32)
+    assert c[1] is not a[1] and torch.equal(c[1], value[csr2csc]) and len(ext_spmm._CSC_CACHE) == 1
+    learned = value.clone().requires_grad_()
+    d = ext_spmm._csc_operands("sum", row, learned, None, csr2csc, True, torch.float32)
+    e = ext_spmm._csc_operands("sum", row, learned, None, csr2csc, True, torch.float32)
+    assert d[1] is not e[1] and not d[1].requires_grad
+    for seed in range(1, 30):                                 # a graph rebuilt every step
+        r2, p2, rc2, v2 = graph(seed)
+        ext_spmm._csc_operands("mean", r2, v2, rc2, p2, True, torch.float32)
+        del r2, p2, rc2, v2
+    gc.collect()
+    assert len(ext_spmm._CSC_CACHE) == 1
+    del row, csr2csc, rowcount, value, a, b, c, m
+    gc.collect()
+    assert len(ext_spmm._CSC_CACHE) == 0

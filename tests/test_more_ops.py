@@ -672,3 +672,41 @@ def test_sparse_product_with_row_strides(backend):
     padded = ext_spmm._aligned_rows(torch.from_numpy(X).to(backend), A.nnz)
     assert padded.shape == (n, K) and padded.stride(0) == 160 and padded.stride(1) == 1
     assert ext_spmm._aligned_rows(wide[:, 5:5 + K], A.nnz).data_ptr() == wide[:, 5:5 + K].data_ptr()
+
+
+@pytest.mark.parametrize("N,K,D", [(1, 1, 1), (7, 3, 5), (100, 40, 256), (515, 256, 128), (1030, 64, 64), (333, 47, 25),
+                                   (1201, 256, 76), (600, 130, 70), (513, 32, 200), (2100, 256, 256)])
+def test_weight_gradient_kernel(N, K, D):
+    """exact_linear_dw_f32 = dY^T . X.  Small integers: every product and sum is
+    exact in fp32, so the result must equal the integer GEMM bit for bit (a
+    wrong fragment, a row counted twice or a column off by one shows); random
+    data within fp32 accumulation error of float64; row strides longer than the
+    used width with NaN in the padding."""
+    rng = np.random.default_rng(N + K + D)
+    dy = rng.integers(-3, 4, (N, K)).astype(np.float32)
+    x = rng.integers(-3, 4, (N, D)).astype(np.float32)
+    assert np.array_equal(e.linear_dw(dy, x), (dy.astype(np.float64).T @ x.astype(np.float64)).astype(np.float32))
+    assert np.array_equal(e.linear_dw(dy, x, ldy=K + 3, ldx=D + 9), (dy.astype(np.float64).T @ x.astype(np.float64)).astype(np.float32))
+    dy, x = rng.standard_normal((N, K)).astype(np.float32), rng.standard_normal((N, D)).astype(np.float32)
+    want = dy.astype(np.float64).T @ x.astype(np.float64)
+    bound = np.abs(dy).astype(np.float64).T @ np.abs(x).astype(np.float64)
+    assert (np.abs(e.linear_dw(dy, x) - want) <= 1e-5 * bound + 1e-30).all()
+
+
+def test_weight_gradient_limits():
+    assert e.linear_dw(np.zeros((0, 4), np.float32), np.zeros((0, 6), np.float32)).tolist() == [[0.0] * 6] * 4
+    assert e.emu().exact_linear_dw_f32(None, 4, None, 3, 5, 4, 6, None, None) == -3      # ldx < D
+
+
+def test_linear_backward_uses_the_weight_gradient_kernel(backend):
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator().manual_seed(9)
+    N, K, D = 16500, 48, 100
+    dy, x = torch.randn(N, K, generator=g).to(backend), torch.randn(N, D, generator=g).to(backend)
+    got = bf.weight_gradient(dy, x)
+    want = dy.double().t().mm(x.double())
+    assert got.dtype == torch.float32 and (got.double() - want).abs().max().item() <= 1e-5 * dy.abs().double().t().mm(x.abs().double()).max().item()
+    wide = torch.randn(N, D + 28, generator=g).to(backend)
+    assert torch.allclose(bf.weight_gradient(dy, wide[:, 3:3 + D]), dy.t().mm(wide[:, 3:3 + D]), rtol=1e-4, atol=1e-2)
+    small = torch.randn(100, 5).to(backend)
+    assert torch.equal(bf.weight_gradient(small, small), small.t().mm(small))       # short batches keep the library GEMM
