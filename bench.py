@@ -3,13 +3,19 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (the op-level microbenchmark configuration): an fp32 activation [169343, 256] ~ N(0,1)
-resident in HBM.  One step = quantize_activation + dequantize_activation at
+Workload (the op-level microbenchmark configuration): fp32 activations [169343, 256] ~ N(0,1)
+in device memory.  One step = quantize_activation + dequantize_activation at
 every bit width {1,2,4,8}: per-row min/range + stochastic-rounding quantise +
 bit-pack (internal Philox noise), then unpack + dequantise with the bf16
 scale/min -- eight kernel launches through the C ABI of libexact_hip.so on
-preallocated buffers.  `value` is the algorithmic bytes of a step divided by
-its time.  Prints ONE JSON line on stdout; progress goes to stderr.
+preallocated buffers.  The steps rotate over four sets of buffers so that no
+step finds its operands in a cache.  `value` is the algorithmic bytes of a
+step divided by its time.  Beside it: every kernel's duration (one HIP event
+pair per launch), the supplied-noise form of the pack kernel, the CPU
+restatement on the host's cores, and -- from a child process -- the other
+kernels of the path and epochs/s of the three full-batch model configurations
+with the roofline fraction of an epoch.  Prints ONE JSON line on stdout;
+progress goes to stderr.
 """
 import argparse
 import json
@@ -180,19 +186,21 @@ def main(argv=None):
         f"{100 * value / HBM_PEAK_GBS:.1f}% of HBM peak   (one set re-used: {ms_single:.3f} ms/step, {value_single:.1f} GB/s)")
 
     # ---- per-kernel durations, HIP events on the launch stream -----------------
-    # One event pair around EACH launch (what a kernel trace reports per dispatch),
-    # rotating over the buffer sets like the timed region.
+    # `us`: one event pair around a run of 40 launches of the same kernel, rotating
+    # over the buffer sets like the timed region, divided by 40 -- launches of one
+    # stream run one after the other, so this is the kernel's duration plus the
+    # sub-microsecond gap between dispatches, and it is what a kernel trace of this
+    # program reports per dispatch.  `single_launch_us`: an event pair around EACH
+    # launch, which adds the events' own few microseconds.
     def per_launch_us(fn, reps=40):
-        for i in range(4):
-            fn(sets[i % ROTATE])
-        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-        for i, (e0, e1) in enumerate(pairs):
-            e0.record()
-            fn(sets[i % ROTATE])
-            e1.record()
-        benchmarks._sync()
-        ts = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs)
-        return sum(ts) / len(ts), ts[len(ts) // 2]
+        counter = [0]
+
+        def one():
+            fn(sets[counter[0] % ROTATE])
+            counter[0] += 1
+        run_us = benchmarks.event_time(one, reps=reps, warm=4) * 1e6
+        single_us, _ = benchmarks.launch_times(lambda i: fn(sets[i % ROTATE]), reps=reps, warm=0)
+        return run_us, single_us
 
     kernels = []
     for b in BITS:
@@ -203,8 +211,8 @@ def main(argv=None):
                  "(the parity mode; 4 more bytes per element)", lambda s, b=b: pack(b, s, True), algo_bytes_pack(N, G, b, True)),
                 (f"unpack_kernel<bits={b}>", "unpack + dequantise with bf16 scale/min", lambda s, b=b: unpack(b, s),
                  algo_bytes_unpack(N, G, b))):
-            mean_us, median_us = per_launch_us(fn)
-            kernels.append({"kernel": name, "does": does, "us": mean_us, "median_us": median_us, "algo_bytes": nbytes,
+            mean_us, single_us = per_launch_us(fn)
+            kernels.append({"kernel": name, "does": does, "us": mean_us, "single_launch_us": single_us, "algo_bytes": nbytes,
                             "GB/s": nbytes / mean_us / 1e3})
     for k in kernels:
         k["frac_hbm_peak"] = k["GB/s"] / HBM_PEAK_GBS
@@ -218,7 +226,7 @@ def main(argv=None):
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": dom["GB/s"] / HBM_PEAK_GBS, "traffic": traffic,
                 "avg_launch_us": dom["us"], "algo_bytes_per_launch": dom["algo_bytes"],
-                "timing": "one HIP event pair per launch on the launch stream, 40 launches rotating over the buffer sets"}
+                "timing": "HIP events on the launch stream around 40 consecutive launches rotating over the buffer sets"}
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -229,7 +237,7 @@ def main(argv=None):
             log(f"cpu baseline failed: {type(e).__name__}: {e}")
 
     del sets[1:], noise
-    torch.cuda.empty_cache()
+    benchmarks._trim()
     if args.no_extras:
         extras = {}
     elif args.extras_in_process:
@@ -254,6 +262,8 @@ def main(argv=None):
         "single_buffer_set": {"value": value_single, "ms_per_step": ms_single,
                               "note": "every step re-reads the same 173 MB input (smaller than the 256 MB memory-side cache)"},
         "epochs_per_s": {k: v.get("epochs_per_s") for k, v in extras.items() if isinstance(v, dict) and k.startswith("cfg")},
+        "epoch_roofline": {k: v.get("epoch_roofline") for k, v in extras.items()
+                           if isinstance(v, dict) and k.startswith("cfg") and "epoch_roofline" in v},
         "roofline": roofline, "cpu_baseline": cpu, "kernels": kernels, "pack_geometry": geometry, "extras": extras,
     }
     print(json.dumps(result), flush=True)

@@ -39,6 +39,22 @@ def event_time(fn, reps=20, warm=3):
     return e0.elapsed_time(e1) / reps * 1e-3
 
 
+def launch_times(fn, reps=40, warm=4):
+    """(mean, median) microseconds of fn(i), one HIP event pair around EACH call
+    on the current stream -- what a kernel trace reports per dispatch, without
+    the overlap of back-to-back launches."""
+    for i in range(warm):
+        fn(i)
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for i, (e0, e1) in enumerate(pairs):
+        e0.record()
+        fn(i)
+        e1.record()
+    torch.cuda.synchronize()
+    ts = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs)
+    return sum(ts) / len(ts), ts[len(ts) // 2]
+
+
 def bench_device():
     if not torch.cuda.is_available():
         raise RuntimeError("the benchmarks need a GPU")
@@ -232,6 +248,77 @@ def train_epochs(model, x, adj, labels, train_idx, epochs, warmup, lr=0.01):
     return epochs / dt, float(loss.detach())
 
 
+def epoch_algorithmic_bytes(kind, n, nnz, feat, hidden, classes, layers, bits, kept_frac, batch_norm, idx_bytes=4):
+    """Compulsory memory traffic of one training epoch's kernels on the
+    compression / aggregation path, as a list of (what, bytes): every operand
+    read once and every result written once per kernel, with the library's
+    default fusions (ReLU + dropout (+ batch norm) + quantise in one pass where
+    no projection is configured, projection + quantise in one pass otherwise).
+    Loss, optimiser and the small per-column vectors are left out.  This is
+    the numerator of the epoch's roofline fraction."""
+    f4 = 4 * n
+    widths = [feat] + [hidden] * (layers - 1) + [classes]
+    items = []
+
+    def add(what, nbytes):
+        items.append((what, int(nbytes)))
+
+    def packed(cols):
+        return bits * n * cols / 8 + 8 * n
+
+    def spmm(cols, valued):
+        return (n + 1) * idx_bytes + nnz * (idx_bytes + (4 if valued else 0)) + 2 * f4 * cols
+
+    def kept(cols):                                       # columns of the compressed copy of a [n, cols] activation
+        return int(kept_frac * cols + 0.999) if kept_frac < 1.0 else cols
+
+    for l in range(layers):
+        cin, cout, last = widths[l], widths[l + 1], l == layers - 1
+        needs_dx = l > 0
+        if kind == "gcn":
+            if l == 0 or kept_frac < 1.0:
+                add(f"L{l} quantise input", f4 * cin + packed(kept(cin)))
+            add(f"L{l} GEMM X W^T", f4 * cin + f4 * cout)
+            add(f"L{l} SpMM forward", spmm(cout, True))
+            add(f"L{l} bias add", 2 * f4 * cout)
+            if not last:
+                if batch_norm:
+                    add(f"L{l} quantise batch-norm input", f4 * cout + packed(cout))
+                    add(f"L{l} batch statistics", f4 * cout)
+                add(f"L{l} (norm +) ReLU + dropout + quantise", 2 * f4 * cout + n * cout / 8 + (packed(cout) if kept_frac >= 1.0 else 0))
+                add(f"L{l} backward: mask", 2 * f4 * cout + n * cout / 8)
+                if batch_norm:
+                    add(f"L{l} backward: restore norm input", packed(cout) + f4 * cout)
+                    add(f"L{l} backward: norm column sums", 2 * f4 * cout)
+                    add(f"L{l} backward: norm element-wise", 3 * f4 * cout)
+            add(f"L{l} backward: bias gradient", f4 * cout)
+            add(f"L{l} backward: SpMM transpose", spmm(cout, True))
+            add(f"L{l} backward: restore input", packed(kept(cin)) + f4 * kept(cin))
+            add(f"L{l} backward: dW", f4 * cout + f4 * kept(cin))
+            if needs_dx:
+                add(f"L{l} backward: dX", f4 * cout + f4 * cin)
+        else:
+            add(f"L{l} project + quantise input (shared copy)", f4 * cin + packed(kept(cin)))
+            add(f"L{l} SpMM mean forward", spmm(cin, False))
+            add(f"L{l} project + quantise aggregate", f4 * cin + packed(kept(cin)))
+            add(f"L{l} GEMM lin_l", f4 * cin + f4 * cout)
+            add(f"L{l} GEMM lin_r", f4 * cin + f4 * cout)
+            add(f"L{l} add", 3 * f4 * cout)
+            if not last:
+                add(f"L{l} ReLU + dropout", 2 * f4 * cout + n * cout / 8)
+                add(f"L{l} backward: mask", 2 * f4 * cout + n * cout / 8)
+            add(f"L{l} backward: bias gradient", f4 * cout)
+            for which in ("lin_l", "lin_r"):
+                add(f"L{l} backward: restore {which} input", packed(kept(cin)) + f4 * kept(cin))
+                add(f"L{l} backward: dW {which}", f4 * cout + f4 * kept(cin))
+                if needs_dx:
+                    add(f"L{l} backward: dX {which}", f4 * cout + f4 * cin)
+            if needs_dx:
+                add(f"L{l} backward: SpMM transpose", spmm(cin, True))
+                add(f"L{l} backward: gradient sum", 3 * f4 * cin)
+    return items
+
+
 EPOCH_CONFIGS = {
     # name: (model, N, raw directed edges, features, hidden, classes, layers, bits, kept_frac, batch_norm, dropout)
     "cfg3_gcn_int2": ("gcn", 169343, 1_160_000, 128, 256, 40, 3, 2, 1.0, True, 0.5),
@@ -240,7 +327,7 @@ EPOCH_CONFIGS = {
 }
 
 
-def epoch_benchmark(name, device, log, epochs=10, warmup=3, int32_index=True, scale=1.0):
+def epoch_benchmark(name, device, log, epochs=10, warmup=3, int32_index=True, scale=1.0, with_spmm=True):
     kind, n, edges, feat, hidden, classes, layers, bits, kept_frac, bn, dropout = EPOCH_CONFIGS[name]
     n, edges = int(n * scale), int(edges * scale)
     saved = dict(config.__dict__)
@@ -269,12 +356,23 @@ def epoch_benchmark(name, device, log, epochs=10, warmup=3, int32_index=True, sc
         setup_s = time.perf_counter() - t0
         _reset_peak(device)
         eps, loss = train_epochs(model, x, adj, labels, train_idx, epochs, warmup)
+        parts = epoch_algorithmic_bytes(kind, n, nnz, feat, hidden, classes, layers, bits, kept_frac, bn,
+                                        4 if int32_index else 8)
+        epoch_bytes = sum(b for _, b in parts)
         res = {"epochs_per_s": eps, "ms_per_epoch": 1e3 / eps, "nodes": n, "nnz": nnz, "features": feat,
+               "epoch_roofline": {"bound": "hbm", "algo_bytes_per_epoch": epoch_bytes,
+                                  "achieved": epoch_bytes * eps / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "frac": epoch_bytes * eps / 1e9 / HBM_PEAK_GBS,
+                                  "largest_parts": sorted(parts, key=lambda p: -p[1])[:6],
+                                  "note": "compulsory traffic of the epoch's compression / aggregation / GEMM kernels "
+                                          "(every operand read once, every result written once) over the epoch time"},
                "hidden": hidden, "classes": classes, "layers": layers, "bits": bits, "kept_frac": kept_frac,
                "index_dtype": "int32" if int32_index else "int64", "epochs_timed": epochs, "last_loss": loss,
                "setup_s": setup_s, "peak_mem_GB": _peak_gb(device)}
-        log(f"  {name}: {eps:.2f} epochs/s ({1e3 / eps:.1f} ms/epoch), N={n}, nnz={nnz}, peak {res['peak_mem_GB']:.1f} GB")
-        res["spmm"] = spmm_extras(adj, hidden if kind == "gcn" else feat, log)
+        log(f"  {name}: {eps:.2f} epochs/s ({1e3 / eps:.1f} ms/epoch), N={n}, nnz={nnz}, peak {res['peak_mem_GB']:.1f} GB, "
+            f"compulsory traffic {epoch_bytes / 1e9:.2f} GB/epoch = {100 * res['epoch_roofline']['frac']:.1f}% of HBM peak")
+        if with_spmm:
+            res["spmm"] = spmm_extras(adj, hidden if kind == "gcn" else feat, log)
         return res
     finally:
         config.__dict__.clear()
@@ -343,12 +441,14 @@ def _epoch_main(argv):
     ap.add_argument("--epochs", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--scale", type=float, default=1.0)
+    ap.add_argument("--epochs-only", action="store_true", help="leave out the separate SpMM timings after the epochs")
     args = ap.parse_args(argv)
 
     def log(*a):
         print(*a, file=sys.stderr, flush=True)
 
-    res = epoch_benchmark(args.config, bench_device(), log, epochs=args.epochs, warmup=args.warmup, scale=args.scale)
+    res = epoch_benchmark(args.config, bench_device(), log, epochs=args.epochs, warmup=args.warmup, scale=args.scale,
+                          with_spmm=not args.epochs_only)
     print(json.dumps(res), flush=True)
 
 

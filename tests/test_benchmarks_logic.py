@@ -24,7 +24,12 @@ def cpu_harness(backend, monkeypatch):
             fn()
         return (time.perf_counter() - t0) / reps
 
+    def wall_launch_times(fn, reps=2, warm=0):
+        t = wall_time(lambda: fn(0), reps=2) * 1e6
+        return t, t
+
     monkeypatch.setattr(bm, "event_time", wall_time)
+    monkeypatch.setattr(bm, "launch_times", wall_launch_times)
     monkeypatch.setattr(bm, "_sync", lambda: None)
     monkeypatch.setattr(bm, "_reset_peak", lambda d: None)
     monkeypatch.setattr(bm, "_peak_gb", lambda d: 0.0)
@@ -89,7 +94,11 @@ def test_bench_py_emits_the_contract_line(cpu_harness, capsys):
     assert r["unit"] == "GB/s" and r["n_gpus"] == 1 and r["vs_baseline"] is None and "workload" in r["config"]
     assert set(r["roofline"]) >= {"bound", "achieved", "peak", "unit", "frac", "traffic"} and r["roofline"]["peak"] == 8000.0
     assert set(r["cpu_baseline"]) >= {"value", "unit", "cores", "kind", "sample"} and r["cpu_baseline"]["kind"] == "port"
-    assert len(r["kernels"]) == 8 and set(r["epochs_per_s"]) == set(bm.EPOCH_CONFIGS)
+    assert len(r["kernels"]) == 12 and set(r["epochs_per_s"]) == set(bm.EPOCH_CONFIGS)
+    assert sum("supplied noise" in k["kernel"] for k in r["kernels"]) == 4          # the parity mode beside the headline
+    assert r["single_buffer_set"]["value"] > 0 and r["config"]["buffer_sets"] == 4
+    for name in bm.EPOCH_CONFIGS:
+        assert 0 < r["epoch_roofline"][name]["frac"] and r["epoch_roofline"][name]["algo_bytes_per_epoch"] > 0
     with pytest.raises(SystemExit):
         bench.main(["--gpus", "2"])
 
