@@ -120,43 +120,14 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_kernel(const float* __restrict_
                                                         const float* __restrict__ R, int64_t N, int D,
                                                         int k, float* __restrict__ out) {
   HIP_DYNAMIC_SHARED(float, Rl)  // [kFwdDChunk][NT * 32]
-  constexpr int KP = NT * kTile;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const int half = lane >> 5;
   const int l32 = lane & 31;
   const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kTile;
-  const int64_t my_row = (row0 + l32 < N) ? row0 + l32 : N - 1;
-  const float* xrow = X + my_row * D;
 
   floatx16 acc[NT];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
-
-  for (int dc = 0; dc < D; dc += kFwdDChunk) {
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < kFwdDChunk * KP; idx += kBlock) {
-      const int rr = idx / KP, cc = idx - rr * KP;
-      Rl[idx] = (dc + rr < D && cc < k) ? R[static_cast<int64_t>(dc + rr) * k + cc] : 0.f;
-    }
-    __syncthreads();
-    const int dlim = (D - dc < kFwdDChunk) ? D - dc : kFwdDChunk;
-    for (int kb = 0; kb < dlim; kb += 2 * VEC) {
-      const int ks = kb + VEC * half;  // this lane's k-slice inside the chunk
-      float a[VEC];
-      load_k_slice<VEC>(xrow, dc + ks, D, a);
-#pragma unroll
-      for (int t = 0; t < VEC; ++t) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const float b = Rl[(ks + t) * KP + nt * kTile + l32];
-          acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b, acc[nt], 0, 0, 0);
-        }
-      }
-    }
-  }
+  rp_fwd_accumulate<VEC, NT>(X, R, N, D, k, Rl, acc);
 
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -310,11 +281,20 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_pack_kernel(const RpPackArgs a)
 }
 
 // out[N, D] = Xr[N, k] . R[D, k]^T;  grid.y tiles D in slabs of NT * 32 columns.
-template <int VEC, int NT>
+// The product is bound by writing [N, D].  In the accumulator layout a store
+// instruction would write 4 bytes per lane; with STAGED (D % 4 == 0, `out`
+// 16-byte aligned) the accumulators leave through a per-wavefront LDS tile of
+// 8 rows instead, from which every lane stores 16 bytes and a store instruction
+// covers whole rows of the slab (up to 512 contiguous bytes each).
+template <int NT>
+constexpr int bwd_stage_pitch() { return NT * kTile + 8; }  // 4 * pitch = 32 (mod 64): the two half-waves hit different banks
+
+template <int VEC, int NT, bool STAGED>
 __global__ __launch_bounds__(kBlock) void rp_bwd_kernel(const float* __restrict__ Xr,
                                                         const float* __restrict__ R, int64_t N, int D,
                                                         int k, int kpad, float* __restrict__ out) {
-  HIP_DYNAMIC_SHARED(float, Rl)  // [NT * 32][kpad + 1], odd pitch: conflict-free column reads
+  HIP_DYNAMIC_SHARED(float, Rl)  // [NT * 32][kpad + 1], odd pitch: conflict-free column reads; then the staging tiles
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
   const int pitch = kpad + 1;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
@@ -351,13 +331,37 @@ __global__ __launch_bounds__(kBlock) void rp_bwd_kernel(const float* __restrict_
     }
   }
 
+  if constexpr (STAGED) {
+    constexpr int PC = bwd_stage_pitch<NT>();
+    constexpr int kQuadsPerRow = NT * kTile / 4;
+    float* Ct = Rl + NT * kTile * pitch + ((-(NT * kTile * pitch)) & 3) + wave * (8 * PC);  // 16-byte aligned [8][PC]
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    const int cj = dbase + nt * kTile + l32;
+    for (int g = 0; g < 4; ++g) {  // rows 8 g .. 8 g + 7 of the wavefront's 32
+      __syncthreads();             // the tile's previous contents have been read
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int64_t rr = row0 + 8 * (v / 4) + 4 * half + (v % 4);
-      if (rr < N && cj < D) __builtin_nontemporal_store(acc[nt][v], out + rr * D + cj);
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Ct[(4 * half + r) * PC + nt * kTile + l32] = acc[nt][4 * g + r];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int f = j * kWave + lane;
+        const int tr = f / kQuadsPerRow, tq = f - tr * kQuadsPerRow;
+        const int64_t rr = row0 + 8 * g + tr;
+        const int cj = dbase + 4 * tq;
+        const floatx4 q = *reinterpret_cast<const floatx4*>(Ct + tr * PC + 4 * tq);
+        if (rr < N && cj < D) __builtin_nontemporal_store(q, reinterpret_cast<floatx4*>(out + rr * D + cj));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int cj = dbase + nt * kTile + l32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t rr = row0 + 8 * (v / 4) + 4 * half + (v % 4);
+        if (rr < N && cj < D) __builtin_nontemporal_store(acc[nt][v], out + rr * D + cj);
+      }
     }
   }
 }
@@ -400,12 +404,19 @@ static int rp_fwd_pack_launch(const RpPackArgs& a, hipStream_t s) {
 template <int VEC>
 static int rp_bwd_launch(const float* Xr, const float* R, int64_t N, int D, int k, float* out, hipStream_t s) {
   const int kpad = ((k + 2 * VEC - 1) / (2 * VEC)) * (2 * VEC);
-  // output slab per workgroup: 128 columns, 64 when R's slab would not fit 64 KB of LDS
-  const int nt = (kpad <= 96) ? 4 : 2;
+  const bool staged = D % 4 == 0 && al16(out);
+  // output slab per workgroup: 128 columns, 64 when R's slab (and the staging tiles) would not fit 64 KB of LDS
+  const int nt = (kpad <= (staged ? 64 : 96)) ? 4 : 2;
   const dim3 grid(static_cast<unsigned>((N + 127) / 128), static_cast<unsigned>((D + nt * kTile - 1) / (nt * kTile)));
-  const size_t lds = static_cast<size_t>(nt) * kTile * (kpad + 1) * sizeof(float);
-  if (nt == 4) hipLaunchKernelGGL((rp_bwd_kernel<VEC, 4>), grid, dim3(kBlock), lds, s, Xr, R, N, D, k, kpad, out);
-  else hipLaunchKernelGGL((rp_bwd_kernel<VEC, 2>), grid, dim3(kBlock), lds, s, Xr, R, N, D, k, kpad, out);
+  const size_t r_floats = static_cast<size_t>(nt) * kTile * (kpad + 1);
+  const size_t lds = sizeof(float) * (r_floats + 3 + (staged ? (kBlock / kWave) * 8 * (nt * kTile + 8) : 0));
+  if (nt == 4) {
+    if (staged) hipLaunchKernelGGL((rp_bwd_kernel<VEC, 4, true>), grid, dim3(kBlock), lds, s, Xr, R, N, D, k, kpad, out);
+    else hipLaunchKernelGGL((rp_bwd_kernel<VEC, 4, false>), grid, dim3(kBlock), lds, s, Xr, R, N, D, k, kpad, out);
+  } else {
+    if (staged) hipLaunchKernelGGL((rp_bwd_kernel<VEC, 2, true>), grid, dim3(kBlock), lds, s, Xr, R, N, D, k, kpad, out);
+    else hipLaunchKernelGGL((rp_bwd_kernel<VEC, 2, false>), grid, dim3(kBlock), lds, s, Xr, R, N, D, k, kpad, out);
+  }
   return launch_status();
 }
 

@@ -3,7 +3,7 @@
 // Calls every C-ABI entry point on heap buffers of EXACTLY the documented
 // sizes, so that any out-of-bounds load or store of a kernel is reported by
 // ASan, and compares the results with the C oracle.  Usage:
-//     emu_check [quick|large|full]
+//     emu_check [quick|large|full|rp]
 // `large` adds grids of thousands of workgroups (20011 x 256, a 20000-node
 // graph; minutes); `full` adds the benchmark shapes (169343 x 256 and a
 // 169343-node graph; hours under the sanitizer).
@@ -471,10 +471,20 @@ static void check_dw(int64_t N, int64_t K, int64_t D, int64_t pad, std::mt19937&
     }
 }
 
+static const int64_t kRpShapes[][3] = {{1, 256, 32}, {31, 256, 32}, {200, 256, 32}, {130, 602, 76}, {140, 100, 25}, {129, 256, 64},
+                                       {64, 128, 64}, {77, 50, 15}, {130, 7, 4}, {100, 256, 126}, {33, 256, 128}, {70, 96, 96},
+                                       {133, 97, 13}, {260, 1024, 32}, {2000, 256, 32}, {1700, 100, 25},
+                                       {1100, 602, 76}, {900, 64, 128}, {1537, 50, 15}};
+
 int main(int argc, char** argv) {
   std::setvbuf(stdout, nullptr, _IOLBF, 0);
   const std::string mode = argc > 1 ? argv[1] : "quick";
   std::mt19937 rng(12345);
+  if (mode == "rp") {  // the projection kernels only
+    for (auto& s : kRpShapes) check_rp(s[0], s[1], s[2], rng);
+    std::printf("rp shapes ok (failures so far %d)\n", g_fail);
+    return g_fail != 0;
+  }
   const int64_t shapes[][2] = {{1, 1}, {5, 3}, {37, 25}, {64, 32}, {100, 76}, {33, 40}, {129, 100}, {300, 128},
                                {203, 256}, {61, 602}, {16, 1024}, {19, 520}, {9, 1500}, {7, 2048}, {8, 8}, {3, 4}};
   for (auto& s : shapes)
@@ -492,9 +502,7 @@ int main(int argc, char** argv) {
   check_spmm(130, 130, 6, 30, 120, rng);
   check_spmm(4, 9, 8, 0, 0, rng);
   std::printf("spmm shapes ok (failures so far %d)\n", g_fail);
-  const int64_t rps[][3] = {{1, 256, 32}, {31, 256, 32}, {200, 256, 32}, {130, 602, 76}, {140, 100, 25}, {129, 256, 64},
-                            {64, 128, 64}, {77, 50, 15}, {130, 7, 4}, {100, 256, 126}, {33, 256, 128}};
-  for (auto& s : rps) check_rp(s[0], s[1], s[2], rng);
+  for (auto& s : kRpShapes) check_rp(s[0], s[1], s[2], rng);
   std::printf("rp shapes ok (failures so far %d)\n", g_fail);
   for (int64_t n : {1, 3, 31, 32, 33, 255, 257, 1000, 2049, 4101, 50001}) check_leaky(n, rng);
   check_extra(120, 120, 256, 6, rng);
