@@ -214,8 +214,28 @@ def main(argv=None):
             mean_us, single_us = per_launch_us(fn)
             kernels.append({"kernel": name, "does": does, "us": mean_us, "single_launch_us": single_us, "algo_bytes": nbytes,
                             "GB/s": nbytes / mean_us / 1e3})
+    # What the memory system delivers for each pack kernel's mix of reads and writes: a kernel
+    # without arithmetic that reads the same tensor and writes as many bytes (the library's
+    # traffic probe), timed the same way.  Peak stays the published 8 TB/s; this is the bar
+    # a kernel of this traffic can reach on this device.
+    probe_out = torch.empty(max(16, (N * G // 16) * 16), dtype=torch.uint8, device=dev)
+    probe = {}
+    for b in BITS:
+        def run_probe(s, b=b):
+            rc = L.exact_stream_probe_f32(s["x"].data_ptr(), N * G, 2 * b, probe_out.data_ptr(), sp)
+            assert rc == 0, rc
+        us, _ = per_launch_us(run_probe)
+        nbytes = (N * G // 4096) * 4096 * 4 + (N * G // 4096) * 256 * 2 * b
+        probe[b] = {"us": us, "GB/s": nbytes / us / 1e3}
+        log(f"  traffic probe, {2 * b:2d} bytes out per 64 in     {us:8.1f} us  {nbytes / us / 1e3:8.1f} GB/s  "
+            f"{100 * nbytes / us / 1e3 / HBM_PEAK_GBS:5.1f}% of HBM peak")
+    del probe_out
     for k in kernels:
         k["frac_hbm_peak"] = k["GB/s"] / HBM_PEAK_GBS
+        if k["kernel"].startswith("pack_kernel") and "supplied" not in k["kernel"]:
+            b = int(k["kernel"].split("bits=")[1].split(">")[0])
+            k["traffic_probe_us"] = probe[b]["us"]
+            k["frac_of_traffic_probe"] = probe[b]["us"] / k["us"]
         log(f"  {k['kernel']:<40s} {k['us']:8.1f} us  {k['GB/s']:8.1f} GB/s  {100 * k['frac_hbm_peak']:5.1f}% of HBM peak")
     in_step = [k for k in kernels if "supplied" not in k["kernel"]]
     dom = max(in_step, key=lambda k: k["us"])
@@ -227,6 +247,10 @@ def main(argv=None):
                 "unit": "GB/s", "frac": dom["GB/s"] / HBM_PEAK_GBS, "traffic": traffic,
                 "avg_launch_us": dom["us"], "algo_bytes_per_launch": dom["algo_bytes"],
                 "timing": "HIP events on the launch stream around 40 consecutive launches rotating over the buffer sets"}
+    if "traffic_probe_us" in dom:
+        roofline["traffic_probe"] = {"us": dom["traffic_probe_us"], "frac_of_it": dom["frac_of_traffic_probe"],
+                                     "what": "a kernel without arithmetic that reads the same tensor and writes as many "
+                                             "bytes as this kernel (exact_stream_probe_f32), timed the same way"}
 
     cpu = None
     if not args.no_cpu_baseline:

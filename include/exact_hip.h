@@ -209,6 +209,15 @@ int exact_bn_backward_reduce_f32(const float *dy, const float *x, const float *m
 int exact_col_moments_f32(const float *x, const float *center, int64_t N, int64_t K, float *sum_d, float *sum_d2,
                           void *stream);
 
+/* Measurement aid with no counterpart in the reference: the memory traffic of the
+ * pack kernel without its arithmetic.  Every lane reads 64 bytes of x (n floats,
+ * whole tiles of 4096 floats; the remainder is not touched) and writes
+ * out_bytes (0, 2, 4, 8 or 16: what 1 / 2 / 4 / 8 bits per element make of 16
+ * elements) to `out`, which holds (n / 16) * out_bytes bytes (at least 16).  x
+ * and out 16-byte aligned.  bench.py times it beside the pack kernels: what it
+ * reaches is what the device's memory system delivers for that read/write mix. */
+int exact_stream_probe_f32(const float *x, int64_t n, int out_bytes, void *out, void *stream);
+
 /* Weight gradient of a linear layer, dW[Kout, D] = dY[N, Kout]^T . X[N, D], row-major
  * fp32 with row strides ldy >= Kout and ldx >= D (in elements), N >> Kout, D.
  * Replaces `grad_output.t().mm(input)` of linear_backward (backward_func.cc:88-89)

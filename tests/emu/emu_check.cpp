@@ -420,6 +420,36 @@ static void check_half(int64_t N, int64_t G, int bits, std::mt19937& rng) {
   CHECK(rc == 0, "f16 mask entry points rc=%d", rc);
 }
 
+// the traffic probe: exactly sized buffers, the folded words recomputed here
+static void check_probe(int64_t n, std::mt19937& rng) {
+  std::normal_distribution<float> nd(0.f, 1.f);
+  Buf<float> x(n);
+  for (int64_t i = 0; i < n; ++i) x[i] = nd(rng);
+  const int64_t tiles = n / 4096, lanes = tiles * 256;
+  std::vector<uint32_t> w(lanes);
+  for (int64_t L = 0; L < lanes; ++L) {
+    uint32_t v = 0;
+    for (int u = 0; u < 4; ++u)
+      for (int c = 0; c < 4; ++c) {
+        uint32_t b;
+        std::memcpy(&b, &x[((L / 256) * 1024 + u * 256 + L % 256) * 4 + c], 4);
+        v ^= b;
+      }
+    w[L] = v;
+  }
+  for (int ob : {0, 2, 4, 8, 16}) {
+    const int64_t nb = std::max<int64_t>(16, (n / 16) * ob);
+    Buf<uint8_t> out(nb);
+    std::memset(out.p, 0xA5, nb);
+    CHECK(exact_stream_probe_f32(x.p, n, ob, out.p, nullptr) == 0, "probe rc n=%ld ob=%d", (long)n, ob);
+    bool ok = true;
+    for (int64_t L = 0; L < lanes && ob >= 4; ++L) { uint32_t g; std::memcpy(&g, out.p + L * ob, 4); ok = ok && g == w[L]; }
+    for (int64_t L = 0; L < lanes && ob == 2; ++L) { uint16_t g; std::memcpy(&g, out.p + L * 2, 2); ok = ok && g == (uint16_t)w[L]; }
+    for (int64_t i = lanes * ob; i < nb; ++i) ok = ok && out[i] == 0xA5;
+    CHECK(ok, "probe output differs n=%ld ob=%d", (long)n, ob);
+  }
+}
+
 static void check_colsum(int64_t N, int64_t K, std::mt19937& rng) {
   std::uniform_int_distribution<int> id(-8, 8);
   Buf<float> x(static_cast<size_t>(N * K)), out(static_cast<size_t>(K));
@@ -525,6 +555,8 @@ int main(int argc, char** argv) {
   const int64_t cs[][2] = {{1, 1}, {3, 5}, {7, 47}, {1000, 41}, {4099, 47}, {513, 256}, {33, 602}, {5, 8192}, {20000, 3}};
   for (auto& c : cs) check_colsum(c[0], c[1], rng);
   std::printf("column sums ok (failures so far %d)\n", g_fail);
+  for (int64_t n : {100, 4096, 3 * 4096 + 77, 20 * 4096}) check_probe(n, rng);
+  std::printf("traffic probe ok (failures so far %d)\n", g_fail);
   const int64_t ds[][4] = {{1, 1, 1, 0}, {7, 3, 5, 1}, {100, 40, 256, 0}, {515, 256, 128, 3}, {333, 47, 25, 0}, {1201, 256, 76, 2},
                            {600, 130, 70, 0}, {513, 32, 200, 5}};
   for (auto& d : ds) check_dw(d[0], d[1], d[2], d[3], rng);

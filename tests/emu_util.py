@@ -429,3 +429,17 @@ def linear_dw(dy, x, ldy=None, ldx=None, guard=8, expect_rc=0):
         return None
     assert (out[K * D:] == np.float32(-777.0)).all()
     return out[:K * D].reshape(K, D)
+
+
+def stream_probe(x, out_bytes, guard=32, expect_rc=0):
+    """exact_stream_probe_f32 on a flat fp32 array -> the bytes it wrote."""
+    x = f32(x).reshape(-1)
+    nb = max(16, (x.size // 16) * out_bytes)
+    out = np.full(nb + guard, 0xA5, np.uint8)
+    rc = emu().exact_stream_probe_f32(p(x), x.size, out_bytes, p(out), None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (out[nb:] == 0xA5).all()
+    return out[:nb]
+

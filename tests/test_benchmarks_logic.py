@@ -96,6 +96,8 @@ def test_bench_py_emits_the_contract_line(cpu_harness, capsys):
     assert set(r["cpu_baseline"]) >= {"value", "unit", "cores", "kind", "sample"} and r["cpu_baseline"]["kind"] == "port"
     assert len(r["kernels"]) == 12 and set(r["epochs_per_s"]) == set(bm.EPOCH_CONFIGS)
     assert sum("supplied noise" in k["kernel"] for k in r["kernels"]) == 4          # the parity mode beside the headline
+    assert r["roofline"]["traffic_probe"]["us"] > 0                                  # the same traffic without arithmetic, timed beside it
+    assert sum("frac_of_traffic_probe" in k for k in r["kernels"]) == 4
     assert r["single_buffer_set"]["value"] > 0 and r["config"]["buffer_sets"] == 4
     for name in bm.EPOCH_CONFIGS:
         assert 0 < r["epoch_roofline"][name]["frac"] and r["epoch_roofline"][name]["algo_bytes_per_epoch"] > 0

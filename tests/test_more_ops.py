@@ -710,3 +710,51 @@ def test_linear_backward_uses_the_weight_gradient_kernel(backend):
     assert torch.allclose(bf.weight_gradient(dy, wide[:, 3:3 + D]), dy.t().mm(wide[:, 3:3 + D]), rtol=1e-4, atol=1e-2)
     small = torch.randn(100, 5).to(backend)
     assert torch.equal(bf.weight_gradient(small, small), small.t().mm(small))       # short batches keep the library GEMM
+
+
+def _stream_probe_words(x):
+    """What lane L of the probe folds: the XOR of the bit patterns of its four
+    16-byte loads, quads tile * 1024 + u * 256 + t of the stream."""
+    tiles = x.size // 4096
+    q = x.view(np.uint32)[:tiles * 4096].reshape(tiles, 4, 256, 4)
+    return np.bitwise_xor.reduce(np.bitwise_xor.reduce(q, axis=3), axis=1).reshape(-1)
+
+
+@pytest.mark.parametrize("n", [4096, 3 * 4096 + 77, 10 * 4096])
+def test_stream_probe_reads_every_quad_and_writes_its_share(n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    w = _stream_probe_words(x)
+    lanes = w.size
+    for out_bytes in (2, 4, 8, 16):
+        got = e.stream_probe(x, out_bytes)
+        want = {2: w.astype(np.uint16), 4: w, 8: np.stack([w, ~w], 1), 16: np.stack([w, ~w, w + np.uint32(1), w - np.uint32(1)], 1)}[out_bytes]
+        assert np.array_equal(got[:lanes * out_bytes], np.ascontiguousarray(want).view(np.uint8).reshape(-1)), out_bytes
+        assert (got[lanes * out_bytes:] == 0xA5).all()          # the incomplete last tile writes nothing
+    assert (e.stream_probe(x, 0) == 0xA5).all()                  # read-only form
+
+
+def test_stream_probe_arguments():
+    x = np.zeros(8192, np.float32)
+    assert e.stream_probe(x, 3, expect_rc=-5) is None
+    assert (e.stream_probe(np.zeros(100, np.float32), 4) == 0xA5).all()   # less than one tile: nothing to do
+
+
+@pytest.mark.gpu
+def test_stream_probe_gpu():
+    from exact_amd import _lib
+    dev = torch.device("cuda:0")
+    n = 1000 * 4096 + 5
+    x = torch.randn(n, device=dev)
+    w = _stream_probe_words(x.cpu().numpy())
+    for out_bytes in (0, 2, 4, 8, 16):
+        out = torch.full((max(16, (n // 16) * out_bytes) + 64,), 0xA5, dtype=torch.uint8, device=dev)
+        rc = _lib.lib().exact_stream_probe_f32(x.data_ptr(), n, out_bytes, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        got = out.cpu().numpy()
+        if out_bytes == 4:
+            assert np.array_equal(got[:w.size * 4].view(np.uint32), w)
+        if out_bytes == 2:
+            assert np.array_equal(got[:w.size * 2].view(np.uint16), w.astype(np.uint16))
+        assert (got[w.size * out_bytes:] == 0xA5).all()
+
