@@ -316,7 +316,11 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       const int d0 = 8 * j;
       uint8_t* dst = a.packed + (n / WPT) * a.G + d0;
       if (a.out_vec == 8) {
-        *reinterpret_cast<uint2*>(dst) = make_uint2(w0, w1);
+        // one 8-byte store: written as two struct members, the compiler hoists the
+        // first word's store out of this branch and issues two 4-byte stores
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        const u32x2 both = {w0, w1};
+        *reinterpret_cast<u32x2*>(dst) = both;
       } else if (a.out_vec == 4) {
         *reinterpret_cast<uint32_t*>(dst) = w0;
         if (d0 + 4 < a.G) *reinterpret_cast<uint32_t*>(dst + 4) = w1;
