@@ -457,11 +457,12 @@ def _profile_target(argv=None):
     `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
 
         python -m exact_amd.benchmarks pack --bits 2 --reps 100
-        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy} ...
+        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy,probe} ...
         python -m exact_amd.benchmarks epoch --config cfg3_gcn_int2 --epochs 5
 
     `copy` is a plain device-to-device copy of the same [rows, cols] fp32 tensor
-    (4*rows*cols bytes read, as many written) for calibrating the byte counters."""
+    (4*rows*cols bytes read, as many written) for calibrating the byte counters;
+    `probe` is the library's traffic probe with the pack kernel's byte mix at --bits."""
     import argparse
 
     from . import _lib
@@ -474,7 +475,7 @@ def _profile_target(argv=None):
         return _epoch_main(argv[1:])
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
     ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "relu_dropout_pack", "bn_relu_dropout_pack", "rp_fwd", "rp_bwd",
-                                      "rp_pack", "spmm", "copy"])
+                                      "rp_pack", "spmm", "copy", "probe"])
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--rows", type=int, default=169343)
     ap.add_argument("--cols", type=int, default=256)
@@ -532,6 +533,8 @@ def _profile_target(argv=None):
         "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, out.data_ptr(), sp),
         "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, spmm_x, spmm_reduce),
         "copy": lambda i: out.copy_(x),
+        # the pack kernel's traffic without its arithmetic: 64 bytes in, 2 * bits bytes out per lane
+        "probe": lambda i: L.exact_stream_probe_f32(x.data_ptr(), N * G, 2 * b, out.data_ptr(), sp),
     }
     fn = fns[args.kernel]
     for i in range(args.reps):
