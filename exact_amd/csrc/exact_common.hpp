@@ -36,9 +36,6 @@ __device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
   return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
 }
 
-#ifndef EXACT_PHILOX_ROUNDS
-#define EXACT_PHILOX_ROUNDS 10
-#endif
 struct Philox4 {
   uint32_t x, y, z, w;
 };
@@ -48,7 +45,7 @@ __device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
   constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
   constexpr uint32_t W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
 #pragma unroll
-  for (int r = 0; r < EXACT_PHILOX_ROUNDS; ++r) {
+  for (int r = 0; r < 10; ++r) {
     const uint64_t p0 = static_cast<uint64_t>(M0) * c0;
     const uint64_t p1 = static_cast<uint64_t>(M1) * c2;
     const uint32_t n0 = xor3(static_cast<uint32_t>(p1 >> 32), c1, k0);
