@@ -79,6 +79,40 @@ __device__ __forceinline__ void load_cached8(const float* __restrict__ p, float 
   v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
+// OPT octs of one row segment for a lane, read "row-contiguously": load i of a
+// lane fetches quad (16 bytes) i * lpr + lir of the segment, so that every load
+// instruction covers lpr * 16 contiguous bytes per row (an oct per lane makes
+// the two loads of a lane 16 bytes apart and the instruction skips every other
+// 16 bytes: 5 - 10 % slower).  The lanes 2m and 2m + 1 then hold the two halves
+// of the octs i * lpr / 2 + m (i < 2 OPT) and trade them: the even lane ends up
+// with the octs of even i, the odd lane with those of odd i, i.e. lane lir owns
+// oct (2k + lir % 2) * lpr / 2 + lir / 2 as its k-th -- for a given k the lanes
+// of a row own lpr consecutive octs, so the packed bytes of a row leave in runs
+// of 8 lpr bytes per store instruction.  lpr even; every lane takes part.
+template <int OPT>
+__device__ __forceinline__ int swizzled_oct(int lir, int lpr, int k) {
+  return (2 * k + (lir & 1)) * (lpr >> 1) + (lir >> 1);
+}
+
+template <int OPT>
+__device__ __forceinline__ void load_octs_swizzled(const float* __restrict__ seg, int lpr, int lir, float (&v)[OPT][8]) {
+  f32x4 q[2 * OPT];
+#pragma unroll
+  for (int i = 0; i < 2 * OPT; ++i) q[i] = nt_load4(seg + 4 * (i * lpr + lir));
+  const bool odd = lir & 1;
+#pragma unroll
+  for (int k = 0; k < OPT; ++k) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float even_i = q[2 * k][c], odd_i = q[2 * k + 1][c];  // this lane's half of oct 2k' and of oct 2k' + 1
+      const float send = odd ? even_i : odd_i;
+      const float recv = __int_as_float(dpp_lanes<0xB1>(__float_as_int(send)));  // the neighbour's: lanes 2m <-> 2m + 1
+      v[k][c] = odd ? recv : even_i;       // first half: columns 0..3 of the oct (held by the even lane)
+      v[k][4 + c] = odd ? odd_i : recv;    // second half (held by the odd lane)
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // pack
 // ---------------------------------------------------------------------------
@@ -142,15 +176,35 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   const bool row_ok = n < a.N;
   const int oct_base = blockIdx.y * (lpr * OPT);  // 0 in the fused form
   const int64_t row_off = n * a.G;
+  // which octs of the row segment a lane owns: lane + k * lpr, or the row-contiguous assignment
+  const bool swz = FULL && VEC == 4 && !HALF && lpr >= 2;
+  auto oct_of = [&](int lir, int k) {
+    return oct_base + (swz ? swizzled_oct<OPT>(lir, lpr, k) : lir + k * lpr);
+  };
 
   float v[OPT][8];
   int nv[OPT];
 #pragma unroll
   for (int k = 0; k < OPT; ++k) {
-    const int j = oct_base + lane_in_row + k * lpr;
+    const int j = oct_of(lane_in_row, k);
     const int d0 = 8 * j;
     nv[k] = (row_ok && j < a.opr) ? min(8, a.G - d0) : 0;
-    if (FULL && !row_ok) {
+    if (swz) {
+      // all OPT octs at once, by every lane (the lanes of a pair trade halves): rows past the
+      // end re-read the last row and drop it
+      if constexpr (!HALF) {
+        if (k == 0) {
+          const int64_t n_ld = row_ok ? n : a.N - 1;
+          load_octs_swizzled<OPT>(a.x + n_ld * a.G + 8 * oct_base, lpr, lane_in_row, v);
+          if (!row_ok) {
+#pragma unroll
+            for (int kk = 0; kk < OPT; ++kk)
+#pragma unroll
+              for (int i = 0; i < 8; ++i) v[kk][i] = 0.f;
+          }
+        }
+      }
+    } else if (FULL && !row_ok) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[k][i] = 0.f;
     } else {
@@ -214,7 +268,7 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
         const int src = wave_first + (q >> 1);  // the thread that produced this quad
         const int half = q & 1;
         const int64_t n_src = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (src >> a.lpr_log2);
-        const int j_src = (src & (lpr - 1)) + k * lpr;
+        const int j_src = oct_of(src & (lpr - 1), k);
         if (n_src < a.N && j_src < a.opr) {
           const f32x4 val = ybuf[(k * kBlock + src) * 2 + half];
           nt_store4(a.y + n_src * a.G + 8 * j_src + 4 * half, val.x, val.y, val.z, val.w);
@@ -260,13 +314,24 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
     }
   }
 
+  // supplied noise: read like x (every lane takes part; rows past the end re-read the last row, their
+  // codes are dropped below)
+  float un[(NOISE_IN && !HALF) ? OPT : 1][8];
+  if constexpr (NOISE_IN && !HALF) {
+    if (swz) load_octs_swizzled<OPT>(a.noise + (row_ok ? n : a.N - 1) * a.G + 8 * oct_base, lpr, lane_in_row, un);
+  }
   uint2 codes[OPT];
 #pragma unroll
   for (int k = 0; k < OPT; ++k) {
-    const int j = oct_base + lane_in_row + k * lpr;
+    const int j = oct_of(lane_in_row, k);
     float u[8];
     if constexpr (NOISE_IN) {
-      if (FULL && !row_ok) {
+      if (swz) {
+        if constexpr (!HALF) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) u[i] = un[k][i];
+        }
+      } else if (FULL && !row_ok) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) u[i] = 0.f;
       } else {
@@ -301,7 +366,7 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   if ((row_local & (WPT - 1)) == 0 && row_ok) {
 #pragma unroll
     for (int k = 0; k < OPT; ++k) {
-      const int j = oct_base + lane_in_row + k * lpr;
+      const int j = oct_of(lane_in_row, k);
       if (j >= a.opr) continue;
       uint32_t w0 = codes[k].x, w1 = codes[k].y;
 #pragma unroll
