@@ -186,7 +186,7 @@ def main(argv=None):
         f"{100 * value / HBM_PEAK_GBS:.1f}% of HBM peak   (one set re-used: {ms_single:.3f} ms/step, {value_single:.1f} GB/s)")
 
     # ---- per-kernel durations, HIP events on the launch stream -----------------
-    # `us`: one event pair around a run of 40 launches of the same kernel, rotating
+    # `us`: one event pair around a run of 40 launches of the same kernel (median of three runs), rotating
     # over the buffer sets like the timed region, divided by 40 -- launches of one
     # stream run one after the other, so this is the kernel's duration plus the
     # sub-microsecond gap between dispatches, and it is what a kernel trace of this
@@ -198,7 +198,8 @@ def main(argv=None):
         def one():
             fn(sets[counter[0] % ROTATE])
             counter[0] += 1
-        run_us = benchmarks.event_time(one, reps=reps, warm=4) * 1e6
+        # the median of three such runs: a single one is now and then disturbed by several microseconds
+        run_us = sorted(benchmarks.event_time(one, reps=reps, warm=4) * 1e6 for _ in range(3))[1]
         single_us, _ = benchmarks.launch_times(lambda i: fn(sets[i % ROTATE]), reps=reps, warm=0)
         return run_us, single_us
 
@@ -246,7 +247,7 @@ def main(argv=None):
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": dom["GB/s"] / HBM_PEAK_GBS, "traffic": traffic,
                 "avg_launch_us": dom["us"], "algo_bytes_per_launch": dom["algo_bytes"],
-                "timing": "HIP events on the launch stream around 40 consecutive launches rotating over the buffer sets"}
+                "timing": "HIP events on the launch stream around 40 consecutive launches rotating over the buffer sets, median of three such runs"}
     if "traffic_probe_us" in dom:
         roofline["traffic_probe"] = {"us": dom["traffic_probe_us"], "frac_of_it": dom["frac_of_traffic_probe"],
                                      "what": "a kernel without arithmetic that reads the same tensor and writes as many "
