@@ -113,6 +113,14 @@ def kernel_extras(x, log):
     out = {}
     N, G = x.shape
     n = N * G
+    # Three copies of the input, used in turn: the [169343, 256] tensor alone fits the 256 MB
+    # memory-side cache, and a kernel timed on one buffer over and over reads it from there.
+    import itertools
+    xs = [x, x.clone(), x.clone()]
+    turn = itertools.count()
+
+    def nx():
+        return xs[next(turn) % 3]
     saved = dict(config.__dict__)
     try:
         config.__dict__.update(QuantizationConfig().__dict__)
@@ -120,34 +128,38 @@ def kernel_extras(x, log):
         mask_bytes = 8 * n + n // 8
         xr = x.clone().requires_grad_()
         y = extq.act_quantized_relu(xr)
-        gy = torch.ones_like(y)
-        t = event_time(lambda: extq.act_quantized_relu(x))
+        gys = [torch.ones_like(y) for _ in range(3)]
+        gy = gys[0]
+
+        def ngy():
+            return gys[next(turn) % 3]
+        t = event_time(lambda: extq.act_quantized_relu(nx()))
         out["relu_fwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
-        t = event_time(lambda: torch.autograd.grad(y, xr, gy, retain_graph=True))
+        t = event_time(lambda: torch.autograd.grad(y, xr, ngy(), retain_graph=True))
         out["relu_bwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
-        t = event_time(lambda: extq.act_quantized_dropout(x, 0.5, True))
+        t = event_time(lambda: extq.act_quantized_dropout(nx(), 0.5, True))
         out["dropout_fwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
         yd = extq.act_quantized_dropout(xr, 0.5, True)
-        t = event_time(lambda: torch.autograd.grad(yd, xr, gy, retain_graph=True))
+        t = event_time(lambda: torch.autograd.grad(yd, xr, ngy(), retain_graph=True))
         out["dropout_bwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes}
-        del y, yd, gy, xr
+        del y, yd, gy, gys, xr
         # --- fused epilogues: ReLU -> dropout (-> INT2 quantise + pack) in one pass --
-        t = event_time(lambda: extq.relu_dropout_fwd(x, 0.5))
+        t = event_time(lambda: extq.relu_dropout_fwd(nx(), 0.5))
         out["relu_dropout_fwd"] = {"us": t * 1e6, "GB/s": mask_bytes / t / 1e9, "algo_bytes": mask_bytes,
                                    "replaces_us": out["relu_fwd"]["us"] + out["dropout_fwd"]["us"]}
         if extq.fusable_width(G):
             fused_bytes = mask_bytes + (2 * n) // 8 + 4 * N
-            t = event_time(lambda: extq.relu_dropout_minmax_pack(x, 0.5, 2))
-            t_pack = event_time(lambda: extq.minmax_pack(x, 2))
+            t = event_time(lambda: extq.relu_dropout_minmax_pack(nx(), 0.5, 2))
+            t_pack = event_time(lambda: extq.minmax_pack(nx(), 2))
             out["relu_dropout_pack_int2"] = {"us": t * 1e6, "GB/s": fused_bytes / t / 1e9, "algo_bytes": fused_bytes,
                                              "replaces_us": out["relu_fwd"]["us"] + out["dropout_fwd"]["us"] + t_pack * 1e6}
             # batch norm folded in: statistics (torch.var_mean) + the one pass, against
             # native_batch_norm + the ReLU / dropout / pack pass
             try:
                 col = torch.ones(G, device=x.device)
-                t_fold = event_time(lambda: extq.bn_relu_dropout_minmax_pack(x, col, col, col, 0.5, 2))
-                t_stats = event_time(lambda: torch.var_mean(x, dim=0, unbiased=False))
-                t_bn = event_time(lambda: torch.ops.aten.native_batch_norm(x, col, col, None, None, True, 0.1, 1e-5))
+                t_fold = event_time(lambda: extq.bn_relu_dropout_minmax_pack(nx(), col, col, col, 0.5, 2))
+                t_stats = event_time(lambda: torch.var_mean(nx(), dim=0, unbiased=False))
+                t_bn = event_time(lambda: torch.ops.aten.native_batch_norm(nx(), col, col, None, None, True, 0.1, 1e-5))
                 out["bn_relu_dropout_pack_int2"] = {"us": t_fold * 1e6, "GB/s": fused_bytes / t_fold / 1e9,
                                                     "algo_bytes": fused_bytes, "stats_us": t_stats * 1e6,
                                                     "replaces_us": t_bn * 1e6 + t * 1e6}
@@ -160,7 +172,7 @@ def kernel_extras(x, log):
         rp_bytes = 4 * N * G + 4 * G * k + 4 * N * k
         flops = 2.0 * N * G * k
         xr_small, _ = ops.input2rp(x, k)
-        t = event_time(lambda: ops.input2rp(x, k))
+        t = event_time(lambda: ops.input2rp(nx(), k))
         out["rp_fwd"] = {"us": t * 1e6, "GB/s": rp_bytes / t / 1e9, "TFLOP/s": flops / t / 1e12,
                          "mfma_frac_of_fp32_peak": flops / t / 1e12 / FP32_MFMA_PEAK_TFLOPS, "algo_bytes": rp_bytes}
         t = event_time(lambda: ops.rp2input(xr_small, x.shape, R))
@@ -169,12 +181,12 @@ def kernel_extras(x, log):
         # compress = project + quantise + pack of the reduced tensor, and back
         config.kept_frac, config.rp_matrix_source = 0.125, (lambda D_, k_, device: R)
         q = ops.quantize_activation(xr_small, None)
-        t = event_time(lambda: ops.quantize_activation(ops.input2rp(x, k)[0], None))
+        t = event_time(lambda: ops.quantize_activation(ops.input2rp(nx(), k)[0], None))
         out["rp_compress_int2"] = {"us": t * 1e6}
         # the same in one launch: the [N, k] product is quantised in the accumulators
         try:
             fused_bytes = 4 * N * G + 4 * G * k + (2 * N * k) // 8 + 4 * N
-            t_one = event_time(lambda: ops.project_and_quantize(x, None))
+            t_one = event_time(lambda: ops.project_and_quantize(nx(), None))
             out["rp_pack_int2"] = {"us": t_one * 1e6, "GB/s": fused_bytes / t_one / 1e9, "algo_bytes": fused_bytes,
                                    "replaces_us": t * 1e6}
         except RuntimeError as err:
@@ -489,9 +501,12 @@ def _profile_target(argv=None):
     L = _lib.lib()
     N, G, b = args.rows, args.cols, args.bits
     gen = torch.Generator(device=dev).manual_seed(1234)
-    x = torch.randn((N, G), generator=gen, device=dev)
+    # three input / output sets, used in turn: a launch finds neither its input nor the lines it
+    # writes in the 256 MB memory-side cache (one 173 MB output written over and over would stay there)
+    xs = [torch.randn((N, G), generator=gen, device=dev) for _ in range(3)]
+    outs = [torch.empty_like(xs[0]) for _ in range(3)]
+    x, out = xs[0], outs[0]
     sp = _checks.stream_ptr(x)
-    out = torch.empty_like(x)
     packed = torch.empty(int(L.exact_packed_nbytes(N, G, b)), dtype=torch.int8, device=dev)
     sbf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     mbf = torch.empty(N, dtype=torch.bfloat16, device=dev)
@@ -512,29 +527,29 @@ def _profile_target(argv=None):
         spmm_x = torch.randn((n_nodes, args.width or G), generator=gen, device=dev)
         spmm_reduce = "sum" if kind == "gcn" else "mean"
     fns = {
-        "pack": lambda i: L.exact_minmax_pack_f32(x.data_ptr(), noise.data_ptr() if noise is not None else None, 1,
+        "pack": lambda i: L.exact_minmax_pack_f32(xs[i % 3].data_ptr(), noise.data_ptr() if noise is not None else None, 1,
                                                   i, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),
                                                   mbf.data_ptr(), sp),
         "unpack": lambda i: L.exact_unpack_bf16param_f32(packed.data_ptr(), b, sbf.data_ptr(), mbf.data_ptr(), N, G,
-                                                         out.data_ptr(), sp),
-        "relu": lambda i: L.exact_relu_fwd_f32(x.data_ptr(), N * G, out.data_ptr(), mask.data_ptr(), sp),
-        "dropout": lambda i: L.exact_dropout_fwd_f32(x.data_ptr(), None, 1, i, 0.5, N * G, out.data_ptr(),
+                                                         outs[i % 3].data_ptr(), sp),
+        "relu": lambda i: L.exact_relu_fwd_f32(xs[i % 3].data_ptr(), N * G, outs[i % 3].data_ptr(), mask.data_ptr(), sp),
+        "dropout": lambda i: L.exact_dropout_fwd_f32(xs[i % 3].data_ptr(), None, 1, i, 0.5, N * G, outs[i % 3].data_ptr(),
                                                      mask.data_ptr(), sp),
         "relu_dropout_pack": lambda i: L.exact_relu_dropout_minmax_pack_f32(
-            x.data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G, b, out.data_ptr(), mask.data_ptr(),
+            xs[i % 3].data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G, b, outs[i % 3].data_ptr(), mask.data_ptr(),
             packed.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp),
         "bn_relu_dropout_pack": lambda i: L.exact_bn_relu_dropout_minmax_pack_f32(
-            x.data_ptr(), ones.data_ptr(), ones.data_ptr(), ones.data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G,
-            b, out.data_ptr(), mask.data_ptr(), packed.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp),
-        "rp_pack": lambda i: L.exact_rp_minmax_pack_f32(x.data_ptr(), R.data_ptr(), None, 1, i, N, G, k, b,
+            xs[i % 3].data_ptr(), ones.data_ptr(), ones.data_ptr(), ones.data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G,
+            b, outs[i % 3].data_ptr(), mask.data_ptr(), packed.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp),
+        "rp_pack": lambda i: L.exact_rp_minmax_pack_f32(xs[i % 3].data_ptr(), R.data_ptr(), None, 1, i, N, G, k, b,
                                                         packed_k.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(),
                                                         sp),
-        "rp_fwd": lambda i: L.exact_rp_fwd_f32(x.data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp),
-        "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, out.data_ptr(), sp),
+        "rp_fwd": lambda i: L.exact_rp_fwd_f32(xs[i % 3].data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp),
+        "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, outs[i % 3].data_ptr(), sp),
         "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, spmm_x, spmm_reduce),
-        "copy": lambda i: out.copy_(x),
+        "copy": lambda i: outs[i % 3].copy_(xs[i % 3]),
         # the pack kernel's traffic without its arithmetic: 64 bytes in, 2 * bits bytes out per lane
-        "probe": lambda i: L.exact_stream_probe_f32(x.data_ptr(), N * G, 2 * b, out.data_ptr(), sp),
+        "probe": lambda i: L.exact_stream_probe_f32(xs[i % 3].data_ptr(), N * G, 2 * b, outs[i % 3].data_ptr(), sp),
     }
     fn = fns[args.kernel]
     for i in range(args.reps):
