@@ -562,14 +562,19 @@ int main(int argc, char** argv) {
   for (auto& d : ds) check_dw(d[0], d[1], d[2], d[3], rng);
   std::printf("weight gradient ok (failures so far %d)\n", g_fail);
   if (mode == "large" || mode == "full") {
+    // a line after every group: this part runs for hours under the sanitizer
     for (int bits : {1, 2, 4, 8}) check_quant(20011, 256, bits, bits == 4, rng);
     check_quant(3001, 1024, 2, false, rng);
+    std::printf("  large quant ok (failures so far %d)\n", g_fail);
     check_masks(20011ll * 256 + 3, rng);
+    std::printf("  large masks ok (failures so far %d)\n", g_fail);
     check_spmm(20000, 20000, 256, 14, 5000, rng);
     check_spmm(20000, 20000, 100, 14, 5000, rng);
     check_extra(5000, 5000, 64, 10, rng);
+    std::printf("  large spmm / minmax / sddmm ok (failures so far %d)\n", g_fail);
     check_rp(20011, 256, 32, rng);
     check_rp(5003, 602, 76, rng);
+    std::printf("  large rp ok (failures so far %d)\n", g_fail);
     check_fused(20011, 256, 2, false, rng);
     check_half(20011, 256, 2, rng);
     std::printf("large shapes ok (failures so far %d)\n", g_fail);
