@@ -108,3 +108,24 @@ def test_bn_relu_dropout_pack_equals_the_oracle_chain_on_the_normalised_input(N,
                   norm=(mean, mult, shift))
     normalised = ((x - mean[None, :]) * mult[None, :] + shift[None, :]).astype(F32)   # three fp32 roundings
     _same(got, _chain(normalised, 0.25, bits, act_noise, noise))
+
+
+@pytest.mark.parametrize("folded", [False, True])
+def test_fused_epilogues_at_config_2_size(folded):
+    """Every output of the fused pass on a [169343, 256] activation (INT2, internal Philox
+    streams), with and without the batch norm, bit for bit against the oracle chain."""
+    N, G, bits = 169343, 256, 2
+    print(f"case fused full size folded={folded}", flush=True)
+    rng = np.random.default_rng(2 + folded)
+    x = (rng.standard_normal((N, G), dtype=F32) * F32(2) + F32(0.5)).astype(F32)
+    act_noise = o.philox_noise_flat(31, 16, N * G).reshape(N, G)
+    noise = o.philox_noise_rows(32, 20, N, G)
+    if folded:
+        mean = rng.standard_normal(G).astype(F32)
+        mult = (rng.random(G, dtype=F32) + F32(0.5)).astype(F32)
+        shift = rng.standard_normal(G).astype(F32)
+        got = _launch(x, 0.5, bits, None, None, (31, 16, 32, 20), norm=(mean, mult, shift))
+        x = ((x - mean[None, :]) * mult[None, :] + shift[None, :]).astype(F32)
+    else:
+        got = _launch(x, 0.5, bits, None, None, (31, 16, 32, 20))
+    _same(got, _chain(x, 0.5, bits, act_noise, noise))

@@ -102,3 +102,43 @@ def test_dropout_structure_like_reference_test(cuda):
     a = extq.act_quantized_dropout(torch.ones(8, device=cuda), 0.5, True)
     b = extq.act_quantized_dropout(torch.ones(8, device=cuda), 0.5, True)
     assert (a == 2).all() and (b == 0).all()            # keep = u > p
+
+
+def test_masks_at_config_2_size(cuda):
+    """ReLU, dropout (supplied noise and the internal Philox stream) and the fused pair on
+    every element of a [169343, 256] activation, bit for bit against the oracle."""
+    n, p = 169343 * 256, 0.5
+    print(f"case masks n={n}", flush=True)
+    L = _lib.lib()
+    x = host_randn((n,), 77)
+    tx = dev(x)
+    y = torch.empty_like(tx)
+    mask = torch.full((o.mask_nwords(n) + 4,), 0x5A5A5A5A, dtype=torch.int32, device=cuda)
+    # ReLU forward / backward
+    assert L.exact_relu_fwd_f32(tx.data_ptr(), n, y.data_ptr(), mask.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    want_y, want_mask = o.relu_fwd(x)
+    assert bytes_equal(y, want_y) and bytes_equal(mask[:-4], want_mask) and (mask[-4:] == 0x5A5A5A5A).all()
+    assert L.exact_relu_bwd_f32(tx.data_ptr(), mask.data_ptr(), n, y.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert bytes_equal(y, o.relu_bwd(x, want_mask))
+    # dropout with the internal Philox stream, then with a supplied noise tensor
+    seed, off = 0xFEEDFACE12345678, (5 << 32) + 12
+    assert L.exact_dropout_fwd_f32(tx.data_ptr(), None, seed, off, p, n, y.data_ptr(), mask.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    noise = o.philox_noise_flat(seed, off, n)
+    want_y, want_mask = o.dropout_fwd(x, p, noise)
+    assert bytes_equal(y, want_y) and bytes_equal(mask[:-4], want_mask)
+    tn = dev(noise)
+    assert L.exact_dropout_fwd_f32(tx.data_ptr(), tn.data_ptr(), 0, 0, p, n, y.data_ptr(), mask.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert bytes_equal(y, want_y) and bytes_equal(mask[:-4], want_mask)
+    assert L.exact_dropout_bwd_f32(tx.data_ptr(), mask.data_ptr(), p, n, y.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert bytes_equal(y, o.dropout_bwd(x, want_mask, p))
+    # ReLU -> dropout in one pass = the two oracle operators in a row, one joint mask
+    assert L.exact_relu_dropout_fwd_f32(tx.data_ptr(), tn.data_ptr(), 0, 0, p, n, y.data_ptr(), mask.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    y1, m1 = o.relu_fwd(x)
+    y2, m2 = o.dropout_fwd(y1, p, noise)
+    assert bytes_equal(y, y2) and bytes_equal(mask[:-4], m1 & m2) and (mask[-4:] == 0x5A5A5A5A).all()
