@@ -52,9 +52,15 @@ def test_generated_matrices(cuda):
     assert ((acc / 200 - x).abs().mean() / x.abs().mean()).item() < 0.25
 
 
-@pytest.mark.parametrize("bits", [1, 2, 4, 8])
-@pytest.mark.parametrize("N,D,frac", [(300, 256, 0.125), (1001, 602, 0.125), (515, 100, 0.25), (130, 256, 0.25),
-                                      (77, 50, 0.3), (64, 256, 0.5), (20011, 256, 0.125)])
+def _shape_cases():
+    small = [(300, 256, 0.125), (1001, 602, 0.125), (515, 100, 0.25), (130, 256, 0.25), (77, 50, 0.3), (64, 256, 0.5),
+             (20011, 256, 0.125)]
+    cases = [(N, D, frac, bits) for (N, D, frac) in small for bits in (1, 2, 4, 8)]
+    # the first-layer shapes of the three benchmark configurations at full size, at their own bit width
+    return cases + [(169343, 256, 0.125, 2), (232965, 602, 0.125, 2), (2449029, 100, 0.25, 1)]
+
+
+@pytest.mark.parametrize("N,D,frac,bits", _shape_cases())
 def test_projection_and_quantisation_in_one_launch_against_the_oracle(cuda, N, D, frac, bits):
     """exact_rp_minmax_pack_f32 through the C ABI (input2rp -> quantize_activation,
     ops.py:141-149): packed bytes, scale and min equal the ORACLE's quantiser applied to
