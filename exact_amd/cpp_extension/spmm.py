@@ -130,8 +130,23 @@ def spmm_mean_fw(row, rowptr, col, value, rowcount, colptr, csr2csc, mat):
 # caching, learned or attention edge values) leaves nothing behind.  Per graph
 # there is ONE slot per reduction for the value-dependent part, replaced when
 # the values change; values that require grad change every step and are never
-# kept.
-_CSC_CACHE = WeakIdKeyDictionary()          # csr2csc tensor -> {"row_csc": .., "sum": (tag, w), "mean": (tag, w)}
+# kept.  A slot holds the value tensor it was built from: an address alone does
+# not identify a tensor (the allocator hands a freed block to the next tensor
+# of the same size), but while the slot keeps the tensor alive its block cannot
+# be handed out again, so "same address, same length, same version" then does
+# mean "same values" (another Python wrapper of the same storage shares its
+# version counter).
+_CSC_CACHE = WeakIdKeyDictionary()          # csr2csc tensor -> {"row_csc": .., "sum": (value, version, w), "mean": ..}
+
+
+def _slot_hit(entry, value, has_value):
+    held, version, _ = entry
+    if not has_value:
+        return held is None
+    if held is not value and (held.data_ptr() != value.data_ptr() or held.numel() != value.numel()
+                              or held.stride() != value.stride()):
+        return False
+    return version == value._version and held._version == value._version
 
 
 def _csc_operands(kind, row, value, rowcount, csr2csc, has_value, dtype):
@@ -140,9 +155,8 @@ def _csc_operands(kind, row, value, rowcount, csr2csc, has_value, dtype):
     slot = _CSC_CACHE.get(csr2csc) if cacheable else None
     if slot is not None and slot["row"] != (row.data_ptr(), row.numel()):
         slot = None                                         # the same permutation handed in with other rows
-    tag = (value.data_ptr(), value._version) if has_value else None
-    if slot is not None and kind in slot and slot[kind][0] == tag:
-        return slot["row_csc"], slot[kind][1]
+    if slot is not None and kind in slot and _slot_hit(slot[kind], value, has_value):
+        return slot["row_csc"], slot[kind][2]
     row_csc = slot["row_csc"] if slot is not None else row.index_select(0, csr2csc)
     if kind == "sum":
         w = value.detach().index_select(0, csr2csc) if has_value else None
@@ -152,7 +166,7 @@ def _csc_operands(kind, row, value, rowcount, csr2csc, has_value, dtype):
     if cacheable:
         if slot is None:
             slot = _CSC_CACHE[csr2csc] = {"row": (row.data_ptr(), row.numel()), "row_csc": row_csc, "keep": row}
-        slot[kind] = (tag, w)
+        slot[kind] = (value, value._version, w) if has_value else (None, 0, w)
     return row_csc, w
 
 

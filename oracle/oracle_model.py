@@ -20,6 +20,66 @@ import torch.nn.functional as F
 import exact_oracle as o
 
 
+class _Native:
+    """The element-wise and sparse pieces through the C restatement
+    (exact_oracle.c), which tests/test_oracle.py holds bit for bit to the NumPy
+    functions of the same name: the only way to run a model of benchmark size
+    on the CPU in seconds.  Same signatures as the NumPy module."""
+
+    def __init__(self):
+        import c_oracle
+        self.c = c_oracle
+
+    def quantize_activation(self, x, bits, noise):
+        x2 = np.ascontiguousarray(x, dtype=np.float32).reshape(x.shape[0], -1)
+        mn, mx = self.c.row_minmax(x2)
+        scale = self.c.scale(mn, mx, bits)
+        packed = self.c.pack(x2, mn, scale, bits, noise)
+        return packed, bits, o.bf16_round(scale)[0], o.bf16_round(mn)[0], scale, mn
+
+    def dequantize_activation(self, packed, bits, scale_bf16_bits, min_bf16_bits, shape):
+        scale = (np.asarray(scale_bf16_bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+        mn = (np.asarray(min_bf16_bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+        return self.c.unpack(packed, bits, scale, mn, shape[0], int(np.prod(shape[1:]))).reshape(shape)
+
+    def relu_fwd(self, x):
+        y, mask = self.c.relu_fwd(x)
+        return y.reshape(np.shape(x)), mask
+
+    def relu_bwd(self, dy, mask):
+        return self.c.relu_bwd(dy, mask).reshape(np.shape(dy))
+
+    def dropout_fwd(self, x, p, noise):
+        y, mask = self.c.dropout_fwd(x, p, noise)
+        return y.reshape(np.shape(x)), mask
+
+    def dropout_bwd(self, dy, mask, p):
+        return self.c.dropout_bwd(dy, mask, p).reshape(np.shape(dy))
+
+    def spmm_csr(self, rowptr, col, val, X, reduce="sum"):
+        return self.c.spmm_csr(rowptr, col, val, X, reduce)
+
+    def spmm_sum_bw(self, row, colptr, csr2csc, val, dY):
+        v = None if val is None else np.asarray(val, dtype=np.float32)[csr2csc]
+        return self.c.spmm_csr(colptr, row[csr2csc], v, dY, "sum")
+
+    def spmm_mean_bw(self, row, rowcount, colptr, csr2csc, val, dY):
+        r = row[csr2csc]
+        cnt = np.maximum(np.asarray(rowcount)[r].astype(np.float32), np.float32(1.0))
+        w = (np.float32(1.0) / cnt).astype(np.float32) if val is None else \
+            (np.asarray(val, dtype=np.float32)[csr2csc] / cnt).astype(np.float32)
+        return self.c.spmm_csr(colptr, r, w, dY, "sum")
+
+
+_impl = o          # the module whose functions the classes below call: the NumPy oracle, or _Native()
+
+
+def use_native(on=True):
+    """Route quantise / dequantise / masks / SpMM through the C restatement."""
+    global _impl
+    _impl = _Native() if on else o
+
+
 class Ctx:
     """What the reference keeps in exact.config plus the random sources."""
 
@@ -29,11 +89,11 @@ class Ctx:
     def quantize(self, x):                                   # ops.py:69-83
         x2 = x.detach().numpy().reshape(x.shape[0], -1)
         u = self.noise(x2.shape).numpy()
-        packed, bits, sbf, mbf, _, _ = o.quantize_activation(x2, self.bits, u)
+        packed, bits, sbf, mbf, _, _ = _impl.quantize_activation(x2, self.bits, u)
         return packed, bits, sbf, mbf
 
     def dequantize(self, q, shape):                          # ops.py:86-98
-        return torch.from_numpy(o.dequantize_activation(q[0], q[1], q[2], q[3], tuple(shape)))
+        return torch.from_numpy(_impl.dequantize_activation(q[0], q[1], q[2], q[3], tuple(shape)))
 
     def compress(self, x):                                   # ops.py:141-149
         if self.kept_frac < 1.0:
@@ -86,26 +146,26 @@ class QBatchNormFn(torch.autograd.Function):
 class ReLUFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x):
-        y, mask = o.relu_fwd(x.detach().numpy())
+        y, mask = _impl.relu_fwd(x.detach().numpy())
         ctx.mask = mask
         return torch.from_numpy(y)
 
     @staticmethod
     def backward(ctx, g):
-        return torch.from_numpy(o.relu_bwd(g.contiguous().numpy(), ctx.mask))
+        return torch.from_numpy(_impl.relu_bwd(g.contiguous().numpy(), ctx.mask))
 
 
 class DropoutFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, c, x, p):
         u = c.noise(tuple(x.shape)).numpy()
-        y, mask = o.dropout_fwd(x.detach().numpy(), p, u)
+        y, mask = _impl.dropout_fwd(x.detach().numpy(), p, u)
         ctx.mask, ctx.p = mask, p
         return torch.from_numpy(y)
 
     @staticmethod
     def backward(ctx, g):
-        return None, torch.from_numpy(o.dropout_bwd(g.contiguous().numpy(), ctx.mask, ctx.p)), None
+        return None, torch.from_numpy(_impl.dropout_bwd(g.contiguous().numpy(), ctx.mask, ctx.p)), None
 
 
 class Graph:
@@ -123,15 +183,15 @@ class SpMMFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, g, x, reduce):
         ctx.g, ctx.reduce = g, reduce
-        return torch.from_numpy(o.spmm_csr(g.rowptr, g.col, g.value, x.detach().numpy(), reduce))
+        return torch.from_numpy(_impl.spmm_csr(g.rowptr, g.col, g.value, x.detach().numpy(), reduce))
 
     @staticmethod
     def backward(ctx, grad):
         g, dY = ctx.g, grad.contiguous().numpy()
         if ctx.reduce == "sum":
-            out = o.spmm_sum_bw(g.row, g.colptr, g.csr2csc, g.value, dY)
+            out = _impl.spmm_sum_bw(g.row, g.colptr, g.csr2csc, g.value, dY)
         else:
-            out = o.spmm_mean_bw(g.row, g.rowcount, g.colptr, g.csr2csc, g.value, dY)
+            out = _impl.spmm_mean_bw(g.row, g.rowcount, g.colptr, g.csr2csc, g.value, dY)
         return None, torch.from_numpy(out), None
 
 

@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 import torch
 
+import c_oracle as co
 import exact_oracle as o
 from exact_amd import _lib, ops
 from exact_amd.conf import config
@@ -158,11 +159,19 @@ def test_full_size_properties(cuda, bits):
     config.noise_source = FixedNoise([torch.full_like(x, 0.5)])
     packed2 = extq.pack_single_precision(xh, m32, x.max(1).values, s32, bits, True)
     assert torch.equal(packed2, packed)
-    # rows sampled across the tensor, compared with the oracle bit for bit
-    rows = torch.arange(0, N - 8, 8 * 1009, device=cuda)[:16]
-    for r in rows.tolist():
-        xs, us = x[r:r + 8].cpu().numpy(), u[r:r + 8].cpu().numpy()
-        want = o.quantize_activation(xs, bits, us)[0][:-1]
-        wpt = 8 // bits
-        got = packed[(r // wpt) * G:(r // wpt) * G + want.size].cpu().numpy().view(np.uint8)
-        assert np.array_equal(got, want)
+    # every packed byte against the oracle's packer (the C restatement, which the CPU tests hold bit for bit to
+    # the NumPy one), given the row statistics verified above
+    want = co.pack(x.cpu().numpy(), m32.cpu().numpy(), s32.cpu().numpy(), bits, u.cpu().numpy())
+    got = packed.cpu().numpy().view(np.uint8)
+    assert got.size == want.size and np.array_equal(got, want)
+    # and for the internal Philox stream
+    config.noise_source = None
+    seed, off = 0x5EEDF00D1234, (7 << 32) + 12
+    nb = int(_lib.lib().exact_packed_nbytes(N, G, bits))
+    p2 = torch.empty(nb, dtype=torch.int8, device=cuda)
+    s2, m2 = torch.empty(N, device=cuda), torch.empty(N, device=cuda)
+    rc = _lib.lib().exact_minmax_pack_f32(x.data_ptr(), None, seed, off, N, G, bits, p2.data_ptr(), s2.data_ptr(),
+                                          m2.data_ptr(), None, None, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(s2, s32) and torch.equal(m2, m32)
+    want = co.pack(x.cpu().numpy(), m32.cpu().numpy(), s32.cpu().numpy(), bits, None, seed, off)
+    assert np.array_equal(p2.cpu().numpy().view(np.uint8), want)

@@ -148,6 +148,26 @@ def test_transpose_operands_are_kept_per_graph_and_die_with_it():
     value.mul_(2.0)                                           # same storage, new version: the slot is rebuilt
     c = ext_spmm._csc_operands("sum", row, value, None, csr2csc, True, torch.float32)
     assert c[1] is not a[1] and torch.equal(c[1], value[csr2csc]) and len(ext_spmm._CSC_CACHE) == 1
+    # two different tensors of version 0 at the same address (what the caching allocator produces when edge
+    # weights are recomputed every step): the address must not be taken for the tensor
+    import numpy as np
+    buf = np.random.default_rng(0).random(400, dtype=np.float32)
+    first = torch.from_numpy(buf)
+    f = ext_spmm._csc_operands("sum", row, first, None, csr2csc, True, torch.float32)
+    assert torch.equal(f[1], first[csr2csc])
+    assert ext_spmm._CSC_CACHE[csr2csc]["sum"][0] is first     # held: its block cannot be reused while the slot lives
+    kept_first = first.clone()
+    del first
+    ext_spmm._CSC_CACHE[csr2csc]["sum"] = (kept_first, 0, f[1])         # the slot as the allocator would leave it
+    buf[:] = np.random.default_rng(1).random(400, dtype=np.float32)
+    second = torch.from_numpy(buf)
+    assert second._version == 0
+    s2 = ext_spmm._csc_operands("sum", row, second, None, csr2csc, True, torch.float32)
+    assert torch.equal(s2[1], second[csr2csc]) and not torch.equal(s2[1], f[1])
+    alias = second.detach()                                    # another wrapper of the same storage does hit
+    s3 = ext_spmm._csc_operands("sum", row, alias, None, csr2csc, True, torch.float32)
+    assert s3[1] is s2[1]
+    del kept_first, second, alias, f, s2, s3
     learned = value.clone().requires_grad_()
     d = ext_spmm._csc_operands("sum", row, learned, None, csr2csc, True, torch.float32)
     e = ext_spmm._csc_operands("sum", row, learned, None, csr2csc, True, torch.float32)
