@@ -339,13 +339,18 @@ EPOCH_CONFIGS = {
 }
 
 
-def epoch_benchmark(name, device, log, epochs=10, warmup=3, int32_index=True, scale=1.0, with_spmm=True):
+def epoch_benchmark(name, device, log, epochs=10, warmup=3, int32_index=True, scale=1.0, with_spmm=True,
+                    overrides=None):
     kind, n, edges, feat, hidden, classes, layers, bits, kept_frac, bn, dropout = EPOCH_CONFIGS[name]
     n, edges = int(n * scale), int(edges * scale)
     saved = dict(config.__dict__)
     try:
         config.__dict__.update(QuantizationConfig().__dict__)
         config.activation_compression_bits, config.kept_frac = [bits], kept_frac
+        for field, setting in (overrides or {}).items():
+            if not hasattr(config, field):
+                raise ValueError(f"no config field {field!r}")
+            setattr(config, field, setting)
         t0 = time.perf_counter()
         adj = powerlaw_graph(n, edges, seed=1, device=device)
         if kind == "gcn":
@@ -454,13 +459,17 @@ def _epoch_main(argv):
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--epochs-only", action="store_true", help="leave out the separate SpMM timings after the epochs")
+    ap.add_argument("--set", action="append", default=[], metavar="FIELD=0|1",
+                    help="a boolean field of exact_amd.config to set for the run, e.g. --set sage_single_node=0")
     args = ap.parse_args(argv)
+    overrides = {f: bool(int(v)) for f, v in (item.split("=", 1) for item in args.set)}
 
     def log(*a):
         print(*a, file=sys.stderr, flush=True)
 
     res = epoch_benchmark(args.config, bench_device(), log, epochs=args.epochs, warmup=args.warmup, scale=args.scale,
-                          with_spmm=not args.epochs_only)
+                          with_spmm=not args.epochs_only, overrides=overrides)
+    res["config_overrides"] = overrides
     print(json.dumps(res), flush=True)
 
 

@@ -52,6 +52,21 @@ _EXTRA_FIELDS = {
     # instead of native_batch_norm, so results agree with the separate layers to
     # rounding (about 1e-6 relative), not bit for bit.  Needs fuse_epilogue.
     "fold_batch_norm": True,
+    # QSAGEConv as one autograd node (lin_l(aggregate(x)) + lin_r(x)) that keeps
+    # what the reference's chain of three nodes keeps.  False: the chain.
+    "sage_single_node": True,
+    # In that node's backward, A^T (dY W_l) is computed as (A^T dY) W_l when the
+    # layer narrows (out < in): the sparse product runs at the smaller width.
+    # Same numbers up to the order of fp32 sums; nothing kept changes.
+    "sage_reassociate_backward": True,
+    # In that node's forward, with a projection (kept_frac < 1) and k + out < in,
+    # aggregate x [R | W_l^T] instead of x: the layer's output and the copy lin_l
+    # keeps are both linear in the aggregate.  The kept codes are those of
+    # aggregate(x R) instead of aggregate(x) R: equal up to fp32 rounding ahead
+    # of the quantiser (a stochastic rounding can fall the other way for a value
+    # within an ulp of a boundary), so results agree with the chain to rounding,
+    # not bit for bit.
+    "sage_aggregate_projected": True,
     # Time the alternative work splits of the pack kernel (1, 2 or 4 column
     # groups per lane) the first time a large activation of a new (width, bits)
     # is compressed on a GPU, and keep the fastest.  Results do not depend on it.

@@ -15,8 +15,8 @@ from torch.nn import Parameter
 from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCN2Conv, GCNConv, GENConv, GraphConv, SAGEConv, glorot
-from .ops import (bn_relu_dropout, consumer_bits, project_and_quantize, qbatch_norm, qelu, qlinear,
-                  quantize_activation, relu_dropout, take_compressed)
+from .ops import (CompressedActivation, bn_relu_dropout, consumer_bits, project_and_quantize, qbatch_norm, qelu,
+                  qlinear, qsage, quantize_activation, relu_dropout, take_compressed)
 from .qsheme import QScheme
 from .spmm import QMatmul, qmatmul
 
@@ -139,8 +139,33 @@ class QSAGEConv(SAGEConv):
             return quantized, randmat
         return quantize_activation(x, self.scheme), None
 
+    def _as_one_node(self, x, adj_t):
+        """The whole layer through ops.qsage where that node applies (one fp32
+        2-D input for both sides, root weight, sum or mean aggregation, edge
+        values without a gradient), else None."""
+        if not (config.sage_single_node and self.training and self.root_weight and x.dim() == 2
+                and x.dtype == torch.float32 and not torch.is_autocast_enabled()
+                and self.msg_and_aggr_func.reduce in ("sum", "mean")):
+            return None
+        rowptr, col, value = adj_t.csr()
+        if value is not None and (value.requires_grad or value.dtype != torch.float32):
+            return None
+        st = adj_t.storage
+        if x.requires_grad:
+            graph = (st.row(), rowptr, col, value, st.rowcount(), st.colptr(), st.csr2csc())
+        else:
+            graph = (st._row, rowptr, col, value, st._rowcount, st._colptr, st._csr2csc)
+        quantized, randmat = self._shared_copy(x)
+        shared = CompressedActivation.adopt(x, quantized, randmat)
+        return qsage.apply(x, self.lin_l.weight, self.lin_l.bias, self.lin_r.weight, graph,
+                           self.msg_and_aggr_func.reduce, shared, self.lin_l.scheme)
+
     def forward(self, x, edge_index, size=None):
         same_both_sides = isinstance(x, torch.Tensor)
+        if same_both_sides:
+            out = self._as_one_node(x, edge_index)
+            if out is not None:
+                return F.normalize(out, p=2.0, dim=-1) if self.normalize else out
         x_l, x_r = (x, x) if same_both_sides else x
         quantized, randmat = self._shared_copy(x_l) if (same_both_sides and self.training) else (None, None)
         out = self.lin_l(self.message_and_aggregate(edge_index, (x_l, x_r), quantized=quantized, randmat=randmat))

@@ -381,6 +381,110 @@ class qspmm_mean(Function):
         return None, None, None, grad_value, None, None, None, None, grad_mat, None, None, None
 
 
+def _restored_weight_gradient(grad_output, kept):
+    """dW = dY^T X_hat for a compressed X (reference ops.py:163-169).  With a
+    projection, dY^T (X_r R^T) = (dY^T X_r) R^T: the [N, D] decompressed input
+    is never formed; only the order of the fp32 sums differs."""
+    if kept.randmat is None:
+        return ext_backward_func.weight_gradient(grad_output, kept.restore())
+    x_r = dequantize_activation(kept.quantized, kept.stored_shape)
+    return ext_backward_func.weight_gradient(grad_output, x_r).mm(kept.randmat.t())
+
+
+class qsage(Function):
+    """`lin_l(aggregate(x)) + lin_r(x)` of a GraphSAGE layer as ONE autograd node:
+    the chain qspmm_mean -> qlinear -> qlinear -> add of the reference's
+    QSAGEConv.forward (layers.py:142-149), keeping exactly what that chain keeps
+    for backward (the shared compressed copy of x for lin_r, a compressed copy
+    of the aggregate for lin_l) and returning the same gradients.  Being one
+    node, it may place the linear maps on whichever side of the aggregation
+    moves fewer bytes through the sparse product -- aggregation and the linear
+    maps commute, A (X W) = (A X) W:
+
+      backward   dX = A^T (dY W_l) + dY W_r  is computed as  (A^T dY) W_l + dY W_r
+                 when out < in (config.sage_reassociate_backward): the sparse
+                 product runs at width `out` instead of `in`; same numbers up to
+                 the order of fp32 sums.
+      forward    with a projection (kept_frac < 1) the layer needs aggregate(x)
+                 only as aggregate(x) W_l^T (the output) and aggregate(x) R (the
+                 copy lin_l keeps).  When k + out < in
+                 (config.sage_aggregate_projected) it aggregates x [R | W_l^T] at
+                 that width instead; the kept copy is then the quantised
+                 aggregate of x R, equal to the reference's up to fp32 rounding
+                 ahead of the quantiser.
+
+    The second GEMM of each pair accumulates into the first one's result, so no
+    separate full-tensor addition runs.  `graph` = (row, rowptr, col, value,
+    rowcount, colptr, csr2csc) without a gradient for `value`; `shared` = the
+    CompressedActivation of x that serves lin_r."""
+
+    @staticmethod
+    def forward(ctx, x, weight_l, bias_l, weight_r, graph, reduce, shared, scheme_l):
+        row, rowptr, col, value, rowcount, colptr, csr2csc = graph
+        n, cin = x.shape
+        cout = weight_l.shape[0]
+        k = kept_columns(cin)
+        narrow = (config.sage_aggregate_projected and config.compress_activation and config.kept_frac < 1.0
+                  and not config.simulate and 0 < k and k + cout < cin)
+        if narrow:
+            if scheme_l:
+                scheme_l.note_use()
+            rand_matrix = _projection_matrix(cin, k, x.device, x.dtype).contiguous()
+            width = k + cout
+            # The sparse product gathers rows of x [R | W_l^T]: rows padded to whole 128-byte lines, and an
+            # even number of columns (a zero column if need be) so that it can gather 8 bytes per lane.
+            both = x.new_zeros((cin, (width + 31) // 32 * 32))
+            both[:, :k] = rand_matrix
+            both[:, k:width] = weight_l.detach().t()
+            aggregated = spmm.spmm_csr(rowptr, col, value, x.mm(both)[:, :width + (width & 1)], reduce)
+            quantized = quantize_activation(aggregated[:, :k].contiguous(), None)
+            kept_l = CompressedActivation(quantized, rand_matrix, x.shape, torch.Size((n, k)))
+            out = torch.addmm(aggregated[:, k:width], x, weight_r.t())
+            if bias_l is not None:
+                out += bias_l
+        else:
+            aggregated = spmm.spmm_csr(rowptr, col, value, x, reduce)
+            kept_l = CompressedActivation.compress(aggregated, scheme_l)
+            out = aggregated.mm(weight_l.t()) if bias_l is None else torch.addmm(bias_l, aggregated, weight_l.t())
+            out.addmm_(x, weight_r.t())
+        del aggregated
+        empty_cache(config.empty_cache_threshold)
+        ctx.kept = (kept_l, shared)
+        ctx.weights = (weight_l, weight_r, bias_l is not None)
+        ctx.graph, ctx.reduce = graph, reduce
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        row, rowptr, col, value, rowcount, colptr, csr2csc = ctx.graph
+        weight_l, weight_r, has_bias = ctx.weights
+        (kept_l, shared), ctx.kept = ctx.kept, None
+        grad_output = grad_output.contiguous()
+        has_value = value is not None
+
+        def transpose_product(t):
+            if ctx.reduce == "sum":
+                return spmm.spmm_sum_bw(row, rowptr, col, value, colptr, csr2csc, None, t, has_value, False, True)[1]
+            return spmm.spmm_mean_bw(row, rowptr, col, value, rowcount, colptr, csr2csc, None, t, has_value, False,
+                                     True)[1]
+
+        grad_x = None
+        if ctx.needs_input_grad[0]:
+            cout, cin = weight_l.shape
+            if config.sage_reassociate_backward and cout < cin:
+                grad_x = transpose_product(grad_output).mm(weight_l)
+            else:
+                grad_x = transpose_product(grad_output.mm(weight_l))
+            grad_x.addmm_(grad_output, weight_r)
+        grad_wl = _restored_weight_gradient(grad_output, kept_l) if ctx.needs_input_grad[1] else None
+        del kept_l
+        grad_wr = _restored_weight_gradient(grad_output, shared) if ctx.needs_input_grad[3] else None
+        del shared
+        grad_b = ext_backward_func.column_sums(grad_output) if (has_bias and ctx.needs_input_grad[2]) else None
+        empty_cache(config.empty_cache_threshold)
+        return grad_x, grad_wl, grad_b, grad_wr, None, None, None, None
+
+
 class qelu(Function):
     """ELU that keeps its input compressed (reference ops.py:182-204)."""
 

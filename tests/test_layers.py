@@ -346,6 +346,156 @@ def test_sage_training_loss_tracks_oracle(backend, kept_frac, bits):
         assert abs(loss.item() - loss_o.item()) < 1e-3, (step, loss.item(), loss_o.item())
 
 
+def _sage_layer_case(backend, kept_frac, bits, cin, cout, valued, switches, n=900, seed=5, want_kept=False):
+    """One QSAGEConv forward + backward on both sides -> (product results, oracle results)."""
+    config.kept_frac, config.activation_compression_bits = kept_frac, [bits]
+    for name, on in switches.items():
+        setattr(config, name, on)
+    A = er_graph(n, 9, seed)
+    A[7, :] = 0                                       # a node without neighbours
+    A.eliminate_zeros()
+    adj = SparseTensor.from_scipy(A)
+    if valued:
+        rng = np.random.default_rng(seed)
+        adj = adj.set_value(torch.from_numpy(rng.random(A.nnz).astype(np.float32) + 0.5))
+    else:
+        adj = adj.set_value(None)
+    rowptr, col, value = adj.csr()
+    graph = om.Graph(rowptr.numpy(), col.numpy(), None if value is None else value.numpy())
+    adj = adj.to(backend).fill_cache_()
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n, cin, generator=g)
+    dy = torch.randn(n, cout, generator=g)
+    torch.manual_seed(seed)
+    conv = exact.QSAGEConv(cin, cout).to(backend).train()
+    other = wire_noise(40 + seed)
+    xd = x.clone().to(backend).requires_grad_()
+    y = conv(xd, adj)
+    kept = []
+    if want_kept:                                      # packed codes of lin_l's copy of the aggregate and of the shared copy
+        def walk(fn, seen):
+            if fn is None or fn in seen:
+                return
+            seen.add(fn)
+            if hasattr(fn, "kept") and isinstance(fn.kept, tuple):             # the one-node form
+                kept.extend([fn.kept[0].quantized[0].cpu().clone(), fn.kept[1].quantized[0].cpu().clone()])
+            elif type(fn).__name__ == "qlinearBackward":                      # the chain: lin_l's node, then lin_r's
+                kept.append(fn.kept.quantized[0].cpu().clone())
+            for nxt, _ in fn.next_functions:
+                walk(nxt, seen)
+        walk(y.grad_fn, set())
+        assert len(kept) == 2
+    y.backward(dy.to(backend))
+    mine = [y.detach().cpu(), xd.grad.cpu(), conv.lin_l.weight.grad.cpu(), conv.lin_l.bias.grad.cpu(),
+            conv.lin_r.weight.grad.cpu()] + kept
+    wl, bl, wr = (p.detach().cpu().clone().requires_grad_() for p in (conv.lin_l.weight, conv.lin_l.bias, conv.lin_r.weight))
+    xo = x.clone().requires_grad_()
+    c = om.Ctx(bits, kept_frac, other.noise, other.rademacher)
+    quantized, R, proj_shape = c.compress(xo)                               # layers.py:153-159
+    agg = om.SpMMFn.apply(graph, xo, "mean")
+    yo = om.QLinearFn.apply(c, agg, wl, bl, None, None, None) + om.QLinearFn.apply(c, xo, wr, None, quantized, R, proj_shape)
+    yo.backward(dy)
+    return mine, [yo.detach(), xo.grad, wl.grad, bl.grad, wr.grad]
+
+
+SAGE_FORMS = {
+    "chain": dict(sage_single_node=False),
+    "node": dict(sage_single_node=True, sage_reassociate_backward=False, sage_aggregate_projected=False),
+    "node+backward": dict(sage_single_node=True, sage_reassociate_backward=True, sage_aggregate_projected=False),
+    "node+both": dict(sage_single_node=True, sage_reassociate_backward=True, sage_aggregate_projected=True),
+}
+
+
+@pytest.mark.parametrize("form", list(SAGE_FORMS))
+@pytest.mark.parametrize("kept_frac,bits,cin,cout,valued", [(0.25, 8, 96, 20, False), (0.125, 8, 130, 41, True),
+                                                             (1.0, 8, 64, 24, False), (0.25, 8, 40, 64, False),
+                                                             (0.25, 2, 96, 20, False)])
+def test_sage_layer_in_every_form_matches_the_oracle_chain(backend, form, kept_frac, bits, cin, cout, valued):
+    """QSAGEConv (layers.py:142-149) as the reference's chain of three nodes and
+    as one node, with the linear maps on either side of the aggregation,
+    against the oracle's chain in the reference's order, for narrowing and
+    widening layers, with and without projection and edge values.  Output,
+    input gradient and bias gradient: within 1e-5 of each tensor's largest
+    entry.  The two weight gradients pass through a kept, quantised copy, and
+    the values that reach the quantiser differ in their last bits between any
+    two implementations (order of fp32 sums in the projection and the
+    aggregation), so a stochastic rounding can fall the other way for a value
+    within an ulp of a boundary: their bound allows two such codes on top of
+    the 1e-5."""
+    mine, want = _sage_layer_case(backend, kept_frac, bits, cin, cout, valued, SAGE_FORMS[form])
+    dy_max = 4.5                                                      # |N(0,1)| over 900 x 64 draws stays below
+    k = ops.kept_columns(cin) if kept_frac < 1.0 else cin
+    r_max = k ** -0.5 if kept_frac < 1.0 else 1.0
+    # one code of a kept tensor: its row range / (2^bits - 1); rows of x R or aggregate(x) R stay within +-6 sigma,
+    # sigma^2 <= cin / k * 1.5 for the unit-variance inputs (edge values up to 1.5) of this test
+    step = 12.0 * (1.5 * cin / k) ** 0.5 / (2 ** bits - 1)
+    for name, a, b in zip(("y", "dx", "dW_l", "db_l", "dW_r"), mine, want):
+        scale = b.abs().max().item()
+        err = (a - b).abs().max().item()
+        allowed = 1e-5 * scale + (2 * step * dy_max * r_max if name in ("dW_l", "dW_r") else 0.0)
+        assert err <= allowed, (name, err, scale, allowed)
+
+
+def test_sage_node_against_the_chain_of_this_library(backend):
+    """The one-node forms against the three-node chain of this library on the
+    same inputs and noise.  Without re-association the kept bytes and the
+    parameter gradients are identical bit for bit and only the fused additions
+    move the output and the input gradient by a rounding; moving the linear
+    maps across the aggregation in backward changes the input gradient by
+    rounding only; aggregating the projected input may change a few kept codes
+    of lin_l's copy (values within an ulp of a rounding boundary), nothing else
+    beyond rounding."""
+    results = {}
+    for form, switches in SAGE_FORMS.items():
+        config.__dict__.update(exact.conf.QuantizationConfig().__dict__)
+        results[form] = _sage_layer_case(backend, 0.25, 2, 96, 20, False, switches, want_kept=True)[0]
+    chain = results["chain"]
+    for form in ("node", "node+backward", "node+both"):
+        y, dx, dwl, dbl, dwr, kept_l, shared = results[form]
+        for a, b in ((y, chain[0]), (dx, chain[1])):
+            assert (a - b).abs().max().item() <= 2e-6 * b.abs().max().item(), form
+        assert torch.equal(dbl, chain[3]) and torch.equal(dwr, chain[4]) and torch.equal(shared, chain[6]), form
+        if form != "node+both":
+            assert torch.equal(kept_l, chain[5]) and torch.equal(dwl, chain[2]), form
+        else:
+            differing = (kept_l != chain[5]).sum().item()
+            assert differing <= 2, differing
+            if differing == 0:
+                assert torch.equal(dwl, chain[2])
+
+
+def test_sage_node_keeps_what_the_chain_keeps(backend):
+    """The one-node form holds the same compressed bytes for backward as the
+    chain of the reference: the shared copy of x and lin_l's copy of the
+    aggregate; and where it aggregates the projected input, the sparse product
+    really runs at width k + out."""
+    from exact_amd.cpp_extension import spmm as ext_spmm
+    config.kept_frac, config.activation_compression_bits = 0.25, [2]
+    n, cin, cout = 600, 96, 20
+    adj = SparseTensor.from_scipy(er_graph(n, 8, 2)).set_value(None).to(backend).fill_cache_()
+    x = torch.randn(n, cin).to(backend).requires_grad_()
+    widths = []
+    real = ext_spmm.spmm_csr
+
+    def spy(rowptr, col, value, mat, reduce):
+        widths.append(mat.shape[1])
+        return real(rowptr, col, value, mat, reduce)
+
+    ext_spmm.spmm_csr = spy
+    try:
+        conv = exact.QSAGEConv(cin, cout).to(backend).train()
+        y = conv(x, adj)
+        node = y.grad_fn
+        kept_l, shared = node.kept
+        k = ops.kept_columns(cin)
+        assert kept_l.stored_shape == (n, k) and shared.stored_shape == (n, k)
+        assert kept_l.quantized[0].numel() == 2 * n * k // 8 + 1 and kept_l.randmat.shape == (cin, k)
+        y.sum().backward()
+    finally:
+        ext_spmm.spmm_csr = real
+    assert widths == [k + cout, cout]                  # forward at k + out = 44 instead of 96, backward at out = 20
+
+
 def test_qmodule_conversion_and_state_dict(backend):
     net = GCN(16, 32, 4, 3, dropout=0.3, batch_norm=True)
     ref_keys = list(net.state_dict().keys())
