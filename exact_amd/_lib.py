@@ -66,6 +66,12 @@ SIGNATURES = {
     "exact_elu_bwd_f16": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_rp_fwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_rp_bwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
+    "exact_rp_table_nbytes": (_c_i64, [_c_i64, _c_i64, _c_int]),
+    "exact_rp_prepare_bf16": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
+    "exact_rp_fwd_bf16_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
+    "exact_rp_bwd_bf16_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
+    "exact_rp_minmax_pack_bf16_f32": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_i64,
+                                               _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
 }
 
 _lib = None

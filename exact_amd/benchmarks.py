@@ -165,32 +165,59 @@ def kernel_extras(x, log):
                                                     "replaces_us": t_bn * 1e6 + t * 1e6}
             except RuntimeError as err:          # this entry only; the other timings go on
                 out["bn_relu_dropout_pack_int2"] = {"error": str(err)}
-        # --- random projection 256 -> 32 (kept_frac 0.125), Gaussian N(0, 1/k) --
+        # --- random projection 256 -> 32 (kept_frac 0.125) --------------------------------
+        # Three matrix-core paths: the fp32 instruction, and the bf16 instruction on operands split in three --
+        # for a Gaussian N(0, 1/k) matrix (six products) and for the +-1/sqrt(k) matrix the reference draws
+        # (signs only, three products).  The default entries (rp_fwd, rp_bwd, rp_pack_int2) are what the library
+        # runs by default for the reference's matrix: the signs path.
         k = int(0.125 * G + 0.999)
-        R = torch.randn(G, k, device=x.device) / k ** 0.5
-        config.rp_matrix_source = lambda D_, k_, device: R
         rp_bytes = 4 * N * G + 4 * G * k + 4 * N * k
         flops = 2.0 * N * G * k
-        xr_small, _ = ops.input2rp(x, k)
-        t = event_time(lambda: ops.input2rp(nx(), k))
-        out["rp_fwd"] = {"us": t * 1e6, "GB/s": rp_bytes / t / 1e9, "TFLOP/s": flops / t / 1e12,
-                         "mfma_frac_of_fp32_peak": flops / t / 1e12 / FP32_MFMA_PEAK_TFLOPS, "algo_bytes": rp_bytes}
-        t = event_time(lambda: ops.rp2input(xr_small, x.shape, R))
-        out["rp_bwd"] = {"us": t * 1e6, "GB/s": rp_bytes / t / 1e9, "TFLOP/s": flops / t / 1e12,
-                         "mfma_frac_of_fp32_peak": flops / t / 1e12 / FP32_MFMA_PEAK_TFLOPS, "algo_bytes": rp_bytes}
-        # compress = project + quantise + pack of the reduced tensor, and back
-        config.kept_frac, config.rp_matrix_source = 0.125, (lambda D_, k_, device: R)
-        q = ops.quantize_activation(xr_small, None)
-        t = event_time(lambda: ops.quantize_activation(ops.input2rp(nx(), k)[0], None))
-        out["rp_compress_int2"] = {"us": t * 1e6}
-        # the same in one launch: the [N, k] product is quantised in the accumulators
-        try:
-            fused_bytes = 4 * N * G + 4 * G * k + (2 * N * k) // 8 + 4 * N
-            t_one = event_time(lambda: ops.project_and_quantize(nx(), None))
-            out["rp_pack_int2"] = {"us": t_one * 1e6, "GB/s": fused_bytes / t_one / 1e9, "algo_bytes": fused_bytes,
-                                   "replaces_us": t * 1e6}
-        except RuntimeError as err:
-            out["rp_pack_int2"] = {"error": str(err)}
+        gauss = torch.randn(G, k, device=x.device) / k ** 0.5
+        signs = (2.0 * torch.randint(2, (G, k), device=x.device, dtype=torch.float32) - 1) / k ** 0.5
+        signs._exact_sign_matrix = True
+        from . import _lib
+        from .cpp_extension import _checks
+        L = _lib.lib()
+        sp = _checks.stream_ptr(x)
+        xr_small = torch.empty((N, k), device=x.device)
+        backs = [torch.empty((N, G), device=x.device) for _ in range(3)]
+        pk = torch.empty(extq.packed_nbytes(N, k, 2), dtype=torch.int8, device=x.device)
+        sbf = torch.empty(N, dtype=torch.bfloat16, device=x.device)
+        mbf = torch.empty(N, dtype=torch.bfloat16, device=x.device)
+
+        def rp_entry(t, nbytes):
+            return {"us": t * 1e6, "GB/s": nbytes / t / 1e9, "TFLOP/s": flops / t / 1e12, "algo_bytes": nbytes}
+
+        fused_bytes = 4 * N * G + 4 * G * k + (2 * N * k) // 8 + 4 * N
+        for label, R, mode in (("fp32_gaussian", gauss, 0), ("bf16_split_gaussian", gauss, 1), ("bf16_signs", signs, 2)):
+            tb = extq.rp_table(R, mode) if mode else None     # prepared once per matrix (a 3 us launch), not timed
+            if mode == 0:
+                fw = lambda: L.exact_rp_fwd_f32(nx().data_ptr(), R.data_ptr(), N, G, k, xr_small.data_ptr(), sp)  # noqa: E731
+                bw = lambda: L.exact_rp_bwd_f32(xr_small.data_ptr(), R.data_ptr(), N, G, k, backs[next(turn) % 3].data_ptr(), sp)  # noqa: E731
+                fp = lambda: L.exact_rp_minmax_pack_f32(nx().data_ptr(), R.data_ptr(), None, 1, 4 * next(turn), N, G, k, 2,  # noqa: E731
+                                                        pk.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp)
+            else:
+                fw = lambda: L.exact_rp_fwd_bf16_f32(nx().data_ptr(), tb.data_ptr(), N, G, k, mode, xr_small.data_ptr(), sp)  # noqa: E731
+                bw = lambda: L.exact_rp_bwd_bf16_f32(xr_small.data_ptr(), tb.data_ptr(), N, G, k, mode,  # noqa: E731
+                                                     backs[next(turn) % 3].data_ptr(), sp)
+                fp = lambda: L.exact_rp_minmax_pack_bf16_f32(nx().data_ptr(), tb.data_ptr(), mode, None, 1, 4 * next(turn), N, G,  # noqa: E731
+                                                             k, 2, pk.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp)
+            out[f"rp_fwd_{label}"] = rp_entry(event_time(fw), rp_bytes)
+            out[f"rp_bwd_{label}"] = rp_entry(event_time(bw), rp_bytes)
+            out[f"rp_pack_int2_{label}"] = rp_entry(event_time(fp), fused_bytes)
+        for name in ("rp_fwd", "rp_bwd", "rp_pack_int2"):
+            out[name] = dict(out[f"{name}_bf16_signs"])
+            out[name]["matrix_cores"] = "bf16, signs of the reference's +-1/sqrt(k) matrix"
+        del backs
+        # compress = project + quantise + pack through the Python layer (what a qlinear pays), and back
+        config.kept_frac = 0.125
+        t_two = event_time(lambda: ops.quantize_activation(ops.input2rp(nx(), k)[0], None))
+        out["rp_compress_int2"] = {"us": t_two * 1e6}
+        t_one = event_time(lambda: ops.project_and_quantize(nx(), None))
+        out["rp_pack_int2"]["python_us"] = t_one * 1e6
+        out["rp_pack_int2"]["replaces_us"] = t_two * 1e6
+        q, R, _ = ops.project_and_quantize(x, None)
         t = event_time(lambda: ops.rp2input(ops.dequantize_activation(q, xr_small.shape), x.shape, R))
         out["rp_decompress_int2"] = {"us": t * 1e6}
         for name, v in out.items():
@@ -497,6 +524,9 @@ def _profile_target(argv=None):
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
     ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "relu_dropout_pack", "bn_relu_dropout_pack", "rp_fwd", "rp_bwd",
                                       "rp_pack", "spmm", "copy", "probe"])
+    ap.add_argument("--rp-path", choices=["fp32", "split", "signs"], default="signs",
+                    help="rp_* only: the fp32 matrix-core instruction on a Gaussian matrix, the bf16 instruction on split "
+                         "operands (Gaussian matrix), or on the signs of a +-1/sqrt(k) matrix (the default path)")
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--rows", type=int, default=169343)
     ap.add_argument("--cols", type=int, default=256)
@@ -524,7 +554,12 @@ def _profile_target(argv=None):
     L.exact_minmax_pack_f32(x.data_ptr(), None, 1, 1, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),
                             mbf.data_ptr(), sp)
     k = int(0.125 * G + 0.999)
-    R = torch.randn(G, k, generator=gen, device=dev) / k ** 0.5
+    if args.rp_path == "signs":
+        R = (2.0 * torch.randint(2, (G, k), generator=gen, device=dev, dtype=torch.float32) - 1) / k ** 0.5
+    else:
+        R = torch.randn(G, k, generator=gen, device=dev) / k ** 0.5
+    rp_mode = {"fp32": 0, "split": 1, "signs": 2}[args.rp_path]
+    rp_tb = extq.rp_table(R, rp_mode) if rp_mode else R
     xr = torch.empty((N, k), device=dev)
     packed_k = torch.empty(int(L.exact_packed_nbytes(N, k, b)), dtype=torch.int8, device=dev)
     ones = torch.ones(G, device=dev)
@@ -550,11 +585,16 @@ def _profile_target(argv=None):
         "bn_relu_dropout_pack": lambda i: L.exact_bn_relu_dropout_minmax_pack_f32(
             xs[i % 3].data_ptr(), ones.data_ptr(), ones.data_ptr(), ones.data_ptr(), 0.5, None, 1, 8 * i, None, 1, 8 * i + 4, N, G,
             b, outs[i % 3].data_ptr(), mask.data_ptr(), packed.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(), sp),
-        "rp_pack": lambda i: L.exact_rp_minmax_pack_f32(xs[i % 3].data_ptr(), R.data_ptr(), None, 1, i, N, G, k, b,
-                                                        packed_k.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(),
-                                                        sp),
-        "rp_fwd": lambda i: L.exact_rp_fwd_f32(xs[i % 3].data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp),
-        "rp_bwd": lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, outs[i % 3].data_ptr(), sp),
+        "rp_pack": (lambda i: L.exact_rp_minmax_pack_f32(xs[i % 3].data_ptr(), R.data_ptr(), None, 1, i, N, G, k, b,
+                                                         packed_k.data_ptr(), None, None, sbf.data_ptr(), mbf.data_ptr(),
+                                                         sp)) if rp_mode == 0 else
+                   (lambda i: L.exact_rp_minmax_pack_bf16_f32(xs[i % 3].data_ptr(), rp_tb.data_ptr(), rp_mode, None, 1, i, N, G, k,
+                                                              b, packed_k.data_ptr(), None, None, sbf.data_ptr(),
+                                                              mbf.data_ptr(), sp)),
+        "rp_fwd": (lambda i: L.exact_rp_fwd_f32(xs[i % 3].data_ptr(), R.data_ptr(), N, G, k, xr.data_ptr(), sp)) if rp_mode == 0
+                  else (lambda i: L.exact_rp_fwd_bf16_f32(xs[i % 3].data_ptr(), rp_tb.data_ptr(), N, G, k, rp_mode, xr.data_ptr(), sp)),
+        "rp_bwd": (lambda i: L.exact_rp_bwd_f32(xr.data_ptr(), R.data_ptr(), N, G, k, outs[i % 3].data_ptr(), sp)) if rp_mode == 0
+                  else (lambda i: L.exact_rp_bwd_bf16_f32(xr.data_ptr(), rp_tb.data_ptr(), N, G, k, rp_mode, outs[i % 3].data_ptr(), sp)),
         "spmm": lambda i: ext_spmm.spmm_csr(rowptr, col, value, spmm_x, spmm_reduce),
         "copy": lambda i: outs[i % 3].copy_(xs[i % 3]),
         # the pack kernel's traffic without its arithmetic: 64 bytes in, 2 * bits bytes out per lane

@@ -19,7 +19,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libexact_hip.so")
 
-SOURCES = ["abi.hip", "quant_pack.hip", "quant_unpack.hip", "act_mask.hip", "spmm.hip", "spmm_extra.hip", "rp_gemm.hip", "colsum.hip", "linear_dw.hip", "stream_probe.hip"]
+SOURCES = ["abi.hip", "quant_pack.hip", "quant_unpack.hip", "act_mask.hip", "spmm.hip", "spmm_extra.hip", "rp_gemm.hip", "rp_bf16.hip", "colsum.hip", "linear_dw.hip", "stream_probe.hip"]
 
 # -ffp-contract=off: the quantiser's arithmetic is defined as separately
 #   rounded fp32 operations; kernels that want FMA call fmaf / MFMA explicitly.

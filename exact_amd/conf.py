@@ -31,6 +31,12 @@ _EXTRA_FIELDS = {
     # Distribution of the projection matrix: "rademacher" (+-1/sqrt(k), what the
     # reference draws, ops.py:112-114) or "gaussian" (N(0, 1/k)).
     "rp_distribution": "rademacher",
+    # Matrix-core path of the projection kernels: "bf16" -- the bf16 instruction on
+    # fp32 operands split without error into three bf16 pieces (for the +-c
+    # matrices drawn here, on the signs alone); "fp32" -- the fp32 instruction.
+    # Both are within fp32 rounding of the exact product; they differ from each
+    # other in the last bits.
+    "rp_matrix_cores": "bf16",
     # None: the kernels draw Philox noise keyed by torch's CUDA generator.  A
     # callable (shape, device) -> fp32 uniforms in [0, 1) supplies the noise of
     # stochastic rounding and dropout instead (parity tests feed the oracle and

@@ -173,6 +173,42 @@ def minmax_pack(data, bits, want_fp32=False):
 RP_PACK_MAX_COLUMNS = 128
 
 
+RP_FP32, RP_BF16_SPLIT, RP_BF16_SIGNS = 0, 1, 2      # EXACT_RP_* of the C header (0: the fp32 instruction)
+
+
+def rp_mode(rand_matrix):
+    """Which matrix-core path multiplies by this projection matrix.
+    config.rp_matrix_cores == "fp32": the fp32 instruction.  "bf16" (default):
+    the bf16 instruction on operands split into three bf16 pieces each -- for a
+    matrix that ops._projection_matrix drew as +-c (it marks the tensor) on its
+    signs alone, scaled by c at the end; for any other matrix the general
+    six-product form."""
+    if config.rp_matrix_cores == "fp32":
+        return RP_FP32
+    if config.rp_matrix_cores != "bf16":
+        raise ValueError("config.rp_matrix_cores must be 'bf16' or 'fp32'")
+    return RP_BF16_SIGNS if getattr(rand_matrix, "_exact_sign_matrix", False) else RP_BF16_SPLIT
+
+
+def rp_table(rand_matrix, mode):
+    """The matrix-core operand fragments of a projection matrix for the bf16 entry
+    points (exact_rp_prepare_bf16), built on first use and kept on the tensor
+    object for as long as the matrix is not written to: a layer's forward and
+    backward share one."""
+    kept = getattr(rand_matrix, "_exact_rp_table", None)
+    if kept is not None and kept[0] == (mode, rand_matrix._version, rand_matrix.data_ptr()):
+        return kept[1]
+    D, k = rand_matrix.shape
+    nbytes = int(_lib.lib().exact_rp_table_nbytes(D, k, mode))
+    if nbytes <= 0:
+        raise RuntimeError("the projection kernels take 1 to 128 projected columns")
+    table = torch.empty(nbytes, dtype=torch.uint8, device=rand_matrix.device)
+    rc = _lib.lib().exact_rp_prepare_bf16(ptr(rand_matrix), D, k, mode, ptr(table), _checks.stream_ptr(rand_matrix))
+    _lib.check(rc, "rp_table")
+    rand_matrix._exact_rp_table = ((mode, rand_matrix._version, rand_matrix.data_ptr()), table)
+    return table
+
+
 def rp_minmax_pack(data, rand_matrix, bits):
     """minmax_pack of the projection data[N, D] . rand_matrix[D, k] in one launch:
     the [N, k] product is quantised in the registers that accumulate it
@@ -192,9 +228,15 @@ def rp_minmax_pack(data, rand_matrix, bits):
     scale_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     min_bf = torch.empty(N, dtype=torch.bfloat16, device=dev)
     noise, seed, offset = _noise_for((N, k), dev)
-    rc = _lib.lib().exact_rp_minmax_pack_f32(ptr(data), ptr(rand_matrix), ptr(noise), seed, offset, N, D, k, bits,
-                                             ptr(packed), None, None, ptr(scale_bf), ptr(min_bf),
-                                             _checks.stream_ptr(data))
+    mode = rp_mode(rand_matrix)
+    if mode == RP_FP32:
+        rc = _lib.lib().exact_rp_minmax_pack_f32(ptr(data), ptr(rand_matrix), ptr(noise), seed, offset, N, D, k, bits,
+                                                 ptr(packed), None, None, ptr(scale_bf), ptr(min_bf),
+                                                 _checks.stream_ptr(data))
+    else:
+        rc = _lib.lib().exact_rp_minmax_pack_bf16_f32(ptr(data), ptr(rp_table(rand_matrix, mode)), mode, ptr(noise), seed,
+                                                      offset, N, D, k, bits, ptr(packed), None, None, ptr(scale_bf),
+                                                      ptr(min_bf), _checks.stream_ptr(data))
     _lib.check(rc, "rp_minmax_pack")
     return packed, scale_bf, min_bf
 

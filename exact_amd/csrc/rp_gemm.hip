@@ -18,13 +18,10 @@
 // B-operand lane l = B[l / 32][l % 32]; accumulator register v of lane l is
 // C[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
 
-#include "exact_common.hpp"
+#include "rp_common.hpp"
 
 namespace exact {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
-constexpr int kTile = 32;       // MFMA M and N
 constexpr int kFwdDChunk = 64;  // rows of R staged per LDS fill (forward)
 
 template <int VEC>
@@ -140,144 +137,15 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_kernel(const float* __restrict_
   }
 }
 
-// ---------------------------------------------------------------------------
-// Projection and quantisation in one launch: the [N, k] product stays in the
-// accumulators, where its per-row min / range, the stochastic rounding and the
-// bit-packing of quantize_activation (ops.py:69-83; kernel
-// quantization_cuda_kernel.cu:63-94) are applied to it -- what
-// exact_rp_fwd_f32 followed by exact_minmax_pack_f32 computes, bit for bit,
-// without the [N, k] tensor ever reaching memory.
-//
-// In the accumulator layout a lane holds, per 32-column tile, one column of 16
-// rows: rows 4h .. 4h + 3 of each block of 8 (h = lane / 32).  So the row
-// statistics are butterflies over the 32 lanes of a half-wave; the 2, 4 or 8
-// rows that share a packed byte sit in one lane (8 rows: in the two lanes
-// l and l + 32); and lane l % 32 writes the byte of column l: 32 consecutive
-// bytes per row group.
-//
-// Noise: element (n, d) takes 16-bit half d % 8 of Philox block (d / 8, n), the
-// row stream of the pack kernel.  The 8 lanes that share d / 8 compute the
-// blocks of four rows at a time between them and hand the words round.
-struct RpPackArgs {
-  const float* X;
-  const float* R;
-  const float* noise;  // nullable: [N, k] uniforms
-  uint32_t seed_lo, seed_hi, off_lo, off_hi;
-  int64_t N;
-  int D, k, bits;
-  uint8_t* packed;
-  int64_t pad_index;
-  float* scale_f32;
-  float* min_f32;
-  uint16_t* scale_bf16;
-  uint16_t* min_bf16;
-};
-
+// Projection and quantisation in one launch (the epilogue is rp_quantise_and_pack, rp_common.hpp).
 template <int VEC, int NT, bool NOISE_IN>
 __global__ __launch_bounds__(kBlock) void rp_fwd_pack_kernel(const RpPackArgs a) {
   HIP_DYNAMIC_SHARED(float, Rl)  // [kFwdDChunk][NT * 32]
-  const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
-  const int half = lane >> 5;
-  const int l32 = lane & 31;
   const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kTile;
-  const int k = a.k;
-  const float B = static_cast<float>((1 << a.bits) - 1);
-
   floatx16 acc[NT];
-  rp_fwd_accumulate<VEC, NT>(a.X, a.R, a.N, a.D, k, Rl, acc);
-
-  // The 16 accumulator rows are handled as four blocks of four consecutive rows
-  // (rows 8 * vg + 4 * half + 0 .. 3), the unit in which they share packed bytes;
-  // one block at a time keeps the epilogue within the registers of the main loop.
-  const int i8 = l32 & 7;            // position in the 8-lane group = element of a Philox block
-  const int group_first = lane & ~7;
-#pragma unroll
-  for (int vg = 0; vg < 4; ++vg) {
-    const int64_t rbase = row0 + 8 * vg + 4 * half;  // first of the four rows
-    // ---- row statistics: min / max over the k columns, then scale -----------
-    float mnv[4], sc[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      float lo = __builtin_inff(), hi = -__builtin_inff();
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        if (nt * kTile + l32 < k) {
-          lo = fminf(lo, acc[nt][4 * vg + r]);
-          hi = fmaxf(hi, acc[nt][4 * vg + r]);
-        }
-      }
-      group_minmax(lo, hi, kTile);
-      mnv[r] = lo;
-      const float recip = 1.0f / (hi - lo);  // ops.py:39: reciprocal, then * B -- two roundings
-      sc[r] = recip * B;
-      if (l32 == 0 && rbase + r < a.N) {
-        if (a.scale_f32) a.scale_f32[rbase + r] = sc[r];
-        if (a.min_f32) a.min_f32[rbase + r] = lo;
-        if (a.scale_bf16) a.scale_bf16[rbase + r] = f32_to_bf16_rne(sc[r]);
-        if (a.min_bf16) a.min_bf16[rbase + r] = f32_to_bf16_rne(lo);
-      }
-    }
-
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int cj = nt * kTile + l32;
-      const bool col_ok = cj < k;
-      // ---- noise -------------------------------------------------------------
-      float u[4];
-      if constexpr (NOISE_IN) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) u[r] = (col_ok && rbase + r < a.N) ? a.noise[(rbase + r) * k + cj] : 0.f;
-      } else {
-        // lane i8 of an 8-lane group computes the block of row i8 % 4 (twice over
-        // the group), then every lane fetches the word holding its element
-        const Philox4 mine = philox4x32_10(static_cast<uint32_t>(cj >> 3), static_cast<uint32_t>(rbase + (i8 & 3)),
-                                           a.off_lo, a.off_hi, a.seed_lo, a.seed_hi);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int src = group_first | r;
-          const uint32_t w0 = __shfl(mine.x, src), w1 = __shfl(mine.y, src), w2 = __shfl(mine.z, src),
-                         w3 = __shfl(mine.w, src);
-          const uint32_t lo_pair = (i8 & 2) ? w1 : w0, hi_pair = (i8 & 2) ? w3 : w2;
-          const uint32_t word = (i8 & 4) ? hi_pair : lo_pair;
-          u[r] = u16_to_uniform((i8 & 1) ? (word >> 16) : (word & 0xFFFFu));
-        }
-      }
-      // ---- quantise (quantization_cuda_kernel.cu:89, one rounding per operation) --
-      uint32_t q[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float tq = acc[nt][4 * vg + r] - mnv[r];
-        tq = tq * sc[r];
-        tq = tq + u[r];
-        tq = tq - 0.5f;
-        tq = fmaxf(tq, 0.f);
-        const uint32_t qi = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
-        q[r] = (col_ok && rbase + r < a.N) ? (qi & 0xFFu) : 0u;
-      }
-      // ---- pack: byte (n / wpt) * k + d holds rows n .. n + wpt - 1 of column d ----
-      if (a.bits == 8) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (col_ok && rbase + r < a.N) a.packed[(rbase + r) * k + cj] = static_cast<uint8_t>(q[r]);
-      } else if (a.bits == 4) {
-#pragma unroll
-        for (int r = 0; r < 4; r += 2)
-          if (col_ok && rbase + r < a.N) a.packed[((rbase + r) >> 1) * k + cj] = static_cast<uint8_t>(q[r] | (q[r + 1] << 4));
-      } else if (a.bits == 2) {
-        if (col_ok && rbase < a.N)
-          a.packed[(rbase >> 2) * k + cj] = static_cast<uint8_t>(q[0] | (q[1] << 2) | (q[2] << 4) | (q[3] << 6));
-      } else {
-        const uint32_t nib = q[0] | (q[1] << 1) | (q[2] << 2) | (q[3] << 3);  // rows 4 * half .. 4 * half + 3 of the eight
-        const uint32_t other = __shfl_xor(nib, 32);
-        const uint32_t byte = half ? (other | (nib << 4)) : (nib | (other << 4));
-        const int64_t first = row0 + 8 * vg;
-        // the two half-waves hold the same byte: they take turns storing
-        if (col_ok && first < a.N && (vg & 1) == half) a.packed[(first >> 3) * k + cj] = static_cast<uint8_t>(byte);
-      }
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x == 0) a.packed[a.pad_index] = 0;
+  rp_fwd_accumulate<VEC, NT>(a.X, a.R, a.N, a.D, a.k, Rl, acc);
+  rp_quantise_and_pack<NT, NOISE_IN>(a, acc, row0);
 }
 
 // out[N, D] = Xr[N, k] . R[D, k]^T;  grid.y tiles D in slabs of NT * 32 columns.
@@ -366,10 +234,6 @@ __global__ __launch_bounds__(kBlock) void rp_bwd_kernel(const float* __restrict_
   }
 }
 
-__global__ void rp_zero_byte_kernel(uint8_t* p) { *p = 0; }
-
-static bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-static bool al8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
 
 template <int VEC>
 static int rp_fwd_launch(const float* X, const float* R, int64_t N, int D, int k, float* out, hipStream_t s) {

@@ -131,7 +131,9 @@ def _projection_matrix(D, k, device, dtype):
         return torch.randn((D, k), device=device, dtype=dtype) / k ** 0.5
     # reference ops.py:112-114: Rademacher entries +-1/sqrt(k)
     signs = torch.randint(2, size=(D, k), device=device, dtype=dtype)
-    return (2.0 * signs - 1) / k ** 0.5
+    matrix = (2.0 * signs - 1) / k ** 0.5
+    matrix._exact_sign_matrix = True     # every entry is +-c with one c: the projection kernels may work on the signs alone
+    return matrix
 
 
 RP_KERNEL_MAX_COLUMNS = 128      # k of exact_rp_fwd_f32 / exact_rp_bwd_f32 / exact_rp_minmax_pack_f32
@@ -154,8 +156,14 @@ def input2rp(input, kept_acts):  # noqa: A002
         # accumulators hold: a plain library GEMM, as torch.matmul is in the reference
         return torch.matmul(input, rand_matrix), rand_matrix
     reduced = torch.empty((N, kept_acts), dtype=input.dtype, device=input.device)
-    rc = _lib.lib().exact_rp_fwd_f32(ptr(input), ptr(rand_matrix), N, D, kept_acts, ptr(reduced),
-                                     _checks.stream_ptr(input))
+    mode = ext_quantization.rp_mode(rand_matrix)
+    if mode == ext_quantization.RP_FP32:
+        rc = _lib.lib().exact_rp_fwd_f32(ptr(input), ptr(rand_matrix), N, D, kept_acts, ptr(reduced),
+                                         _checks.stream_ptr(input))
+    else:
+        rc = _lib.lib().exact_rp_fwd_bf16_f32(ptr(input), ptr(ext_quantization.rp_table(rand_matrix, mode)), N, D, kept_acts, mode,
+                                              ptr(reduced),
+                                              _checks.stream_ptr(input))
     _lib.check(rc, "input2rp")
     return reduced, rand_matrix
 
@@ -173,8 +181,14 @@ def rp2input(dim_reduced_input, input_shape, rand_matrix):
     if rand_matrix.shape[1] != k:
         raise RuntimeError("rand_matrix does not match the reduced input")
     full = torch.empty((N, D), dtype=dim_reduced_input.dtype, device=dim_reduced_input.device)
-    rc = _lib.lib().exact_rp_bwd_f32(ptr(dim_reduced_input), ptr(rand_matrix), N, D, k, ptr(full),
-                                     _checks.stream_ptr(dim_reduced_input))
+    mode = ext_quantization.rp_mode(rand_matrix)
+    if mode == ext_quantization.RP_FP32:
+        rc = _lib.lib().exact_rp_bwd_f32(ptr(dim_reduced_input), ptr(rand_matrix), N, D, k, ptr(full),
+                                         _checks.stream_ptr(dim_reduced_input))
+    else:
+        rc = _lib.lib().exact_rp_bwd_bf16_f32(ptr(dim_reduced_input), ptr(ext_quantization.rp_table(rand_matrix, mode)), N, D, k, mode,
+                                              ptr(full),
+                                              _checks.stream_ptr(dim_reduced_input))
     _lib.check(rc, "rp2input")
     return full.view(input_shape)
 

@@ -323,6 +323,40 @@ int exact_rp_minmax_pack_f32(const float *X, const float *R, const float *noise,
                              uint8_t *packed, float *scale_f32, float *min_f32,
                              uint16_t *scale_bf16, uint16_t *min_bf16, void *stream);
 
+/* The same three products on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16,
+ * fp32 accumulate) at fp32 accuracy: every fp32 operand is split, without error,
+ * into three bf16 pieces.  No counterpart in the reference beyond the two
+ * torch.matmul calls of ops.py:117,124 (which ran on TF32 tensor cores there).
+ *   mode EXACT_RP_BF16_SIGNS  R = +-c with one c > 0, the matrix the reference
+ *        draws (ops.py:112-114: (2 * Bernoulli(1/2) - 1) / sqrt(k)); only the
+ *        signs of R are used and the product is scaled once by c = |R[0][0]|.
+ *        The caller vouches that |R| is the same everywhere and not 0.
+ *   mode EXACT_RP_BF16_SPLIT  any R: six bf16 products per fp32 product, the
+ *        neglected ones below 2^-24 of it.
+ * The kernels read R as a TABLE of matrix-core operand fragments, which
+ * exact_rp_prepare_bf16 writes from R[D, k] (row-major fp32) into a buffer of
+ * exact_rp_table_nbytes(D, k, mode) bytes (16-byte aligned) that the caller
+ * allocates and owns; one table serves all three products for as long as R,
+ * D, k and mode stay the same.  exact_rp_table_nbytes returns 0 for shapes
+ * the kernels do not take (k > 128).
+ * exact_rp_minmax_pack_bf16_f32 equals exact_rp_fwd_bf16_f32 followed by
+ * exact_minmax_pack_f32 bit for bit (same mode).  Results differ from the
+ * fp32-matrix-core entry points above in the last bits (different order and
+ * number of roundings); both are within fp32 rounding of the exact product.
+ * Non-finite inputs: a row of X holding inf or NaN gives NaN in that row. */
+#define EXACT_RP_BF16_SPLIT 1
+#define EXACT_RP_BF16_SIGNS 2
+int64_t exact_rp_table_nbytes(int64_t D, int64_t k, int mode);
+int exact_rp_prepare_bf16(const float *R, int64_t D, int64_t k, int mode, void *table, void *stream);
+int exact_rp_fwd_bf16_f32(const float *X, const void *table, int64_t N, int64_t D, int64_t k, int mode,
+                          float *out, void *stream);
+int exact_rp_bwd_bf16_f32(const float *Xr, const void *table, int64_t N, int64_t D, int64_t k, int mode,
+                          float *out, void *stream);
+int exact_rp_minmax_pack_bf16_f32(const float *X, const void *table, int mode, const float *noise,
+                                  uint64_t seed, uint64_t offset, int64_t N, int64_t D, int64_t k,
+                                  int bits, uint8_t *packed, float *scale_f32, float *min_f32,
+                                  uint16_t *scale_bf16, uint16_t *min_bf16, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

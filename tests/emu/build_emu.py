@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 CSRC = os.path.join(ROOT, "exact_amd", "csrc")
 OUT = os.path.join(HERE, "_build")
 CLANG = "/opt/rocm/lib/llvm/bin/clang++"
-SOURCES = ["abi.hip", "quant_pack.hip", "quant_unpack.hip", "act_mask.hip", "spmm.hip", "spmm_extra.hip", "rp_gemm.hip", "colsum.hip", "linear_dw.hip", "stream_probe.hip"]
+SOURCES = ["abi.hip", "quant_pack.hip", "quant_unpack.hip", "act_mask.hip", "spmm.hip", "spmm_extra.hip", "rp_gemm.hip", "rp_bf16.hip", "colsum.hip", "linear_dw.hip", "stream_probe.hip"]
 COMMON = ["-x", "c++", "-std=c++17", "-ffp-contract=off", "-fno-fast-math", "-pthread", "-fPIC",
           "-I", os.path.join(HERE, "include"), "-Wno-unused-value", "-Wno-unknown-attributes"]
 LIB = os.path.join(OUT, "libexact_emu.so")

@@ -169,21 +169,35 @@ static void check_spmm(int64_t M, int64_t ncols, int64_t K, double avg, int64_t 
       }
 }
 
-static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
+// mode 0: the fp32 instruction; EXACT_RP_BF16_SPLIT on a Gaussian matrix; EXACT_RP_BF16_SIGNS on a +-c matrix
+static int rp_fwd_any(int mode, const float* X, const float* R, const void* table, int64_t N, int64_t D, int64_t k, float* out) {
+  return mode == 0 ? exact_rp_fwd_f32(X, R, N, D, k, out, nullptr) : exact_rp_fwd_bf16_f32(X, table, N, D, k, mode, out, nullptr);
+}
+static int rp_bwd_any(int mode, const float* Xr, const float* R, const void* table, int64_t N, int64_t D, int64_t k, float* out) {
+  return mode == 0 ? exact_rp_bwd_f32(Xr, R, N, D, k, out, nullptr) : exact_rp_bwd_bf16_f32(Xr, table, N, D, k, mode, out, nullptr);
+}
+
+static void check_rp_mode(int mode, int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
   std::normal_distribution<float> nd(0.f, 1.f);
   Buf<float> X(N * D), R(D * k), xr(N * k), wxr(N * k), back(N * D), wback(N * D);
   for (int64_t i = 0; i < N * D; ++i) X[i] = nd(rng);
-  for (int64_t i = 0; i < D * k; ++i) R[i] = nd(rng) / std::sqrt((float)k);
+  const float c = 1.f / std::sqrt((float)k);
+  for (int64_t i = 0; i < D * k; ++i) R[i] = mode == EXACT_RP_BF16_SIGNS ? ((rng() & 1) ? c : -c) : nd(rng) * c;
+  // the fragment table of the bf16 paths, on a heap buffer of exactly the documented size
+  const int64_t tbytes = mode == 0 ? 16 : exact_rp_table_nbytes(D, k, mode);
+  CHECK(tbytes > 0 && tbytes % 16 == 0, "rp table size");
+  Buf<uint32_t> table(tbytes / 4);
+  if (mode != 0) CHECK(exact_rp_prepare_bf16(R.p, D, k, mode, table.p, nullptr) == 0, "rp prepare rc");
   oracle_rp_fwd(X.p, R.p, N, D, k, wxr.p);
-  CHECK(exact_rp_fwd_f32(X.p, R.p, N, D, k, xr.p, nullptr) == 0, "rp fwd rc");
+  CHECK(rp_fwd_any(mode, X.p, R.p, table.p, N, D, k, xr.p) == 0, "rp fwd rc");
   double worst = 0, scale = 1e-30;
   for (int64_t i = 0; i < N * k; ++i) { scale = std::max(scale, (double)std::fabs(wxr[i])); worst = std::max(worst, (double)std::fabs(xr[i] - wxr[i])); }
-  CHECK(worst <= 2e-5 * scale, "rp fwd differs N=%ld D=%ld k=%ld: %g of %g", (long)N, (long)D, (long)k, worst, scale);
+  CHECK(worst <= 2e-5 * scale, "rp fwd differs mode=%d N=%ld D=%ld k=%ld: %g of %g", mode, (long)N, (long)D, (long)k, worst, scale);
   oracle_rp_bwd(wxr.p, R.p, N, D, k, wback.p);
-  CHECK(exact_rp_bwd_f32(wxr.p, R.p, N, D, k, back.p, nullptr) == 0, "rp bwd rc");
+  CHECK(rp_bwd_any(mode, wxr.p, R.p, table.p, N, D, k, back.p) == 0, "rp bwd rc");
   worst = 0, scale = 1e-30;
   for (int64_t i = 0; i < N * D; ++i) { scale = std::max(scale, (double)std::fabs(wback[i])); worst = std::max(worst, (double)std::fabs(back[i] - wback[i])); }
-  CHECK(worst <= 2e-5 * scale, "rp bwd differs N=%ld D=%ld k=%ld: %g of %g", (long)N, (long)D, (long)k, worst, scale);
+  CHECK(worst <= 2e-5 * scale, "rp bwd differs mode=%d N=%ld D=%ld k=%ld: %g of %g", mode, (long)N, (long)D, (long)k, worst, scale);
   // projection + quantisation in one launch == the oracle's quantiser on the kernel's own product
   std::uniform_real_distribution<float> ud(0.f, 1.f);
   Buf<float> u(N * k), mn(N), mx(N), sc(N), mn2(N), sc2(N);
@@ -198,12 +212,19 @@ static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
     std::memset(want.p, 0, nb);
     oracle_pack(xr.p, mn.p, sc.p, supplied ? u.p : nullptr, 0x99ull, (7ull << 32) + 16, N, k, bits, want.p);
     std::memset(packed.p, 0xEE, nb);
-    const int rc = exact_rp_minmax_pack_f32(X.p, R.p, supplied ? u.p : nullptr, 0x99ull, (7ull << 32) + 16, N, D, k, bits,
-                                            packed.p, sc2.p, mn2.p, sbf.p, mbf.p, nullptr);
-    CHECK(rc == 0 && std::memcmp(packed.p, want.p, nb) == 0, "rp+pack packed differs N=%ld D=%ld k=%ld bits=%d rc=%d",
-          (long)N, (long)D, (long)k, bits, rc);
-    CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "rp+pack scale/min differ N=%ld k=%ld", (long)N, (long)k);
+    const int rc = mode == 0
+        ? exact_rp_minmax_pack_f32(X.p, R.p, supplied ? u.p : nullptr, 0x99ull, (7ull << 32) + 16, N, D, k, bits,
+                                   packed.p, sc2.p, mn2.p, sbf.p, mbf.p, nullptr)
+        : exact_rp_minmax_pack_bf16_f32(X.p, table.p, mode, supplied ? u.p : nullptr, 0x99ull, (7ull << 32) + 16, N, D, k, bits,
+                                        packed.p, sc2.p, mn2.p, sbf.p, mbf.p, nullptr);
+    CHECK(rc == 0 && std::memcmp(packed.p, want.p, nb) == 0, "rp+pack packed differs mode=%d N=%ld D=%ld k=%ld bits=%d rc=%d",
+          mode, (long)N, (long)D, (long)k, bits, rc);
+    CHECK(std::memcmp(sc2.p, sc.p, N * 4) == 0 && std::memcmp(mn2.p, mn.p, N * 4) == 0, "rp+pack scale/min differ mode=%d N=%ld k=%ld", mode, (long)N, (long)k);
   }
+}
+
+static void check_rp(int64_t N, int64_t D, int64_t k, std::mt19937& rng) {
+  for (int mode : {0, EXACT_RP_BF16_SPLIT, EXACT_RP_BF16_SIGNS}) check_rp_mode(mode, N, D, k, rng);
 }
 
 // LeakyReLU mask, max / min aggregation and the edge-value gradient, against

@@ -405,6 +405,45 @@ inline floatx16_t mfma_f32_32x32x2f32(float a, float b, floatx16_t c, int, int, 
   return c;
 }
 
+// v_mfma_f32_32x32x16_bf16: lane l holds row (A) / column (B) l % 32 and the eight
+// k-slots 8 * (l / 32) .. + 7 as bf16; accumulator layout as for 32x32x2.  The
+// products of two bf16 numbers are exact in fp32; they are added one after the
+// other in fp32 (the hardware's own order is not specified, so tests compare
+// against float64 with a tolerance, and launches that must agree bit for bit
+// with each other go through this same routine).
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+inline floatx16_t mfma_f32_32x32x16_bf16(bf16x8_t a, bf16x8_t b, floatx16_t c, int, int, int) {
+  uint64_t words[4];
+  std::memcpy(&words[0], &a, 16);
+  std::memcpy(&words[2], &b, 16);
+  uint64_t all[4][64];
+  WaveState* w = nullptr;
+  int lane = 0;
+  for (int q = 0; q < 4; ++q) {
+    const int buf = wave_collect(words[q], w, lane);
+    if (w->mask[buf] != ~uint64_t{0}) {
+      std::fprintf(stderr, "hip emulator: MFMA with inactive lanes\n");
+      std::abort();
+    }
+    for (int l = 0; l < 64; ++l) all[q][l] = w->slot[buf][l];
+  }
+  auto element = [&](int base, int l, int e) {      // bf16 element e (0..7) of lane l's operand -> float
+    const uint64_t word = all[base + e / 4][l];
+    const uint32_t bits = static_cast<uint32_t>((word >> (16 * (e % 4))) & 0xFFFFu) << 16;
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+  };
+  const int j = lane % 32;
+  for (int v = 0; v < 16; ++v) {
+    const int i = 8 * (v / 4) + 4 * (lane / 32) + (v % 4);
+    float acc = c[v];
+    for (int kk = 0; kk < 16; ++kk) acc = std::fmaf(element(0, i + 32 * (kk / 8), kk % 8), element(2, j + 32 * (kk / 8), kk % 8), acc);
+    c[v] = acc;
+  }
+  return c;
+}
+
 inline void syncthreads() {
   BlockState* b = g_block;
   const uint64_t my_gen = b->block_gen;
@@ -465,6 +504,11 @@ static inline uint64_t __ballot(bool p) { return hipemu::ballot(p); }
 #define __builtin_amdgcn_update_dpp(old, v, ctrl, rm, bm, bc) hipemu::update_dpp_any((v), (ctrl), (rm), (bm), (bc))
 #define __builtin_amdgcn_bitop3_b32(a, b, c, table) hipemu::bitop3((a), (b), (c), (table))
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) hipemu::mfma_f32_32x32x2f32((a), (b), (c), (x), (y), (z))
+// every active lane of the wavefront arrives before any goes on (a scheduling barrier on the hardware, where the
+// lanes of a wavefront move in lockstep anyway; here the lanes are fibres and must really wait)
+#define __builtin_amdgcn_wave_barrier() ((void)hipemu::ballot(true))
+#define __builtin_amdgcn_fence(order, scope) ((void)0)
+#define __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, x, y, z) hipemu::mfma_f32_32x32x16_bf16((a), (b), (c), (x), (y), (z))
 
 static inline float __fmaf_rn(float a, float b, float c) { return std::fmaf(a, b, c); }
 static inline uint32_t __float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }

@@ -147,17 +147,42 @@ def spmm(rowptr, col, val, X, reduce, idx=np.int64, guard=16):
     return out[:M * K].reshape(M, K)
 
 
-def rp_fwd(X, R, guard=16):
+RP_MODES = {"fp32": 0, "bf16_split": 1, "bf16_signs": 2}
+
+
+def rp_table(R, mode, guard=64):
+    """The operand-fragment table of R for the bf16 entry points (exactly sized, with a guard behind it)."""
+    R = f32(R)
+    if mode == "bf16_signs":
+        assert (np.abs(R) == np.abs(R).max()).all() and np.abs(R).max() > 0, "the signs mode needs a +-c matrix"
+    D, k = R.shape
+    nb = int(emu().exact_rp_table_nbytes(D, k, RP_MODES[mode]))
+    assert nb > 0 and nb % 16 == 0
+    raw = np.full(nb + guard + 16, 0xC3, np.uint8)
+    off = (-raw.ctypes.data) % 16
+    table = raw[off:off + nb + guard]
+    rc = emu().exact_rp_prepare_bf16(p(R), D, k, RP_MODES[mode], p(table), None)
+    assert rc == 0, rc
+    assert (table[nb:] == 0xC3).all()
+    return table
+
+
+def rp_fwd(X, R, guard=16, mode="fp32"):
     X, R = f32(X), f32(R)
     N, D = X.shape
     k = R.shape[1]
     out = np.full(N * k + guard, np.float32(-777.0), np.float32)
-    assert emu().exact_rp_fwd_f32(p(X), p(R), N, D, k, p(out), None) == 0
+    if mode == "fp32":
+        rc = emu().exact_rp_fwd_f32(p(X), p(R), N, D, k, p(out), None)
+    else:
+        table = rp_table(R, mode)          # held until the call has returned
+        rc = emu().exact_rp_fwd_bf16_f32(p(X), p(table), N, D, k, RP_MODES[mode], p(out), None)
+    assert rc == 0, rc
     assert (out[N * k:] == np.float32(-777.0)).all()
     return out[:N * k].reshape(N, k)
 
 
-def rp_minmax_pack(X, R, bits, noise=None, seed=0, offset=0, guard=64, expect_rc=0):
+def rp_minmax_pack(X, R, bits, noise=None, seed=0, offset=0, guard=64, expect_rc=0, mode="fp32"):
     """-> (packed, scale f32, min f32, scale bf16 bits, min bf16 bits) of the projected X."""
     X, R = f32(X), f32(R)
     N, D = X.shape
@@ -167,8 +192,13 @@ def rp_minmax_pack(X, R, bits, noise=None, seed=0, offset=0, guard=64, expect_rc
     s32, m32 = np.full(N + 1, np.float32(-3.0), np.float32), np.full(N + 1, np.float32(-3.0), np.float32)
     sbf, mbf = np.full(N + 1, 0x1234, np.uint16), np.full(N + 1, 0x1234, np.uint16)
     noise = None if noise is None else f32(noise)
-    rc = emu().exact_rp_minmax_pack_f32(p(X), p(R), p(noise), seed, offset, N, D, k, bits, p(packed), p(s32), p(m32),
-                                        p(sbf), p(mbf), None)
+    if mode == "fp32":
+        rc = emu().exact_rp_minmax_pack_f32(p(X), p(R), p(noise), seed, offset, N, D, k, bits, p(packed), p(s32), p(m32),
+                                            p(sbf), p(mbf), None)
+    else:
+        table = rp_table(R, mode)
+        rc = emu().exact_rp_minmax_pack_bf16_f32(p(X), p(table), RP_MODES[mode], p(noise), seed, offset,
+                                                 N, D, k, bits, p(packed), p(s32), p(m32), p(sbf), p(mbf), None)
     assert rc == expect_rc, rc
     if rc != 0:
         return None
@@ -176,12 +206,17 @@ def rp_minmax_pack(X, R, bits, noise=None, seed=0, offset=0, guard=64, expect_rc
     return packed[:nb], s32[:N], m32[:N], sbf[:N], mbf[:N]
 
 
-def rp_bwd(Xr, R, guard=16):
+def rp_bwd(Xr, R, guard=16, mode="fp32"):
     Xr, R = f32(Xr), f32(R)
     N, k = Xr.shape
     D = R.shape[0]
     out = np.full(N * D + guard, np.float32(-777.0), np.float32)
-    assert emu().exact_rp_bwd_f32(p(Xr), p(R), N, D, k, p(out), None) == 0
+    if mode == "fp32":
+        rc = emu().exact_rp_bwd_f32(p(Xr), p(R), N, D, k, p(out), None)
+    else:
+        table = rp_table(R, mode)
+        rc = emu().exact_rp_bwd_bf16_f32(p(Xr), p(table), N, D, k, RP_MODES[mode], p(out), None)
+    assert rc == 0, rc
     assert (out[N * D:] == np.float32(-777.0)).all()
     return out[:N * D].reshape(N, D)
 

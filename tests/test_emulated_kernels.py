@@ -141,37 +141,84 @@ def test_spmm_all_empty_and_single_long_row():
                                       (140, 100, 0.25), (129, 256, 0.25), (64, 128, 0.5), (77, 50, 0.3), (130, 7, 0.5),
                                       (100, 256, 0.49)])
 def test_rp(N, D, frac, dist):
+    """Every matrix-core path of the projection (fp32 instruction; bf16
+    instruction on operands split in three, for any matrix; bf16 on the signs
+    of a +-c matrix) within 1e-5 of the oracle, forward and back."""
     k = o.kept_acts(frac, D)
     rng = np.random.default_rng(N + D)
     R = o.rademacher_matrix(D, k, rng) if dist == "rademacher" else o.gaussian_matrix(D, k, rng)
-    X = rng.standard_normal((N, D)).astype(F32)
+    X = (rng.standard_normal((N, D)) * np.exp(rng.uniform(-6, 6, (N, 1)))).astype(F32)   # rows of very different size
     want = o.input2rp(X, R)
-    got = e.rp_fwd(X, R)
-    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
-    back = e.rp_bwd(got, R)
-    wb = o.rp2input(got, R)
-    np.testing.assert_allclose(back, wb, rtol=1e-5, atol=1e-5 * np.abs(wb).max())
+    for mode in ("fp32", "bf16_split") + (("bf16_signs",) if dist == "rademacher" else ()):
+        got = e.rp_fwd(X, R, mode=mode)
+        row_scale = np.abs(want).max(1, keepdims=True)
+        assert (np.abs(got - want) <= 1e-5 * row_scale + 1e-30).all(), mode
+        back = e.rp_bwd(got, R, mode=mode)
+        wb = o.rp2input(got, R)
+        assert (np.abs(back - wb) <= 1e-5 * np.abs(wb).max(1, keepdims=True) + 1e-30).all(), mode
 
 
+def test_bf16_split_of_an_fp32_number_is_exact():
+    """The identity the bf16 paths rest on: hi = bf16(x), mid = bf16(x - hi),
+    lo = bf16(x - hi - mid) reproduce x exactly (x normal, not within 2^16 of
+    the smallest normal).  Checked here with torch's bf16 rounding, which is
+    the rounding the conversion instruction performs."""
+    import torch
+    g = torch.Generator().manual_seed(0)
+    bits = torch.randint(-2 ** 31, 2 ** 31 - 1, (2_000_000,), generator=g, dtype=torch.int64).to(torch.int32)
+    x = bits.view(torch.float32)
+    x = x[torch.isfinite(x) & (x.abs() > 1e-30) & (x.abs() < 1e38)]
+    hi = x.to(torch.bfloat16).float()
+    r1 = x - hi
+    mid = r1.to(torch.bfloat16).float()
+    r2 = r1 - mid
+    lo = r2.to(torch.bfloat16).float()
+    assert torch.equal(lo, r2)
+    assert torch.equal((hi.double() + mid.double() + lo.double()).float(), x)
+    assert torch.equal(hi.double() + mid.double() + lo.double(), x.double())
+
+
+@pytest.mark.parametrize("N,D,k", [(70, 256, 32), (33, 100, 25), (40, 602, 76), (64, 48, 128)])
+def test_rp_signs_path_on_integers_is_exact(N, D, k):
+    """Small integers times +-1: every term and every partial sum is exact, so
+    the signs path must return c * (integer sum) rounded once -- a wrong
+    fragment, a k-slot paired with the wrong feature or a missed tail shows."""
+    rng = np.random.default_rng(N + D + k)
+    S = (2.0 * rng.integers(0, 2, (D, k)) - 1).astype(F32)
+    c = F32(1.0 / np.sqrt(k))
+    R = (S * c).astype(F32)
+    X = rng.integers(-9, 10, (N, D)).astype(F32) * F32(0.25)
+    exact = X.astype(np.float64) @ S.astype(np.float64)
+    assert np.array_equal(e.rp_fwd(X, R, mode="bf16_signs"), (exact.astype(F32) * c).astype(F32))
+    Xr = rng.integers(-9, 10, (N, k)).astype(F32)
+    exact_b = Xr.astype(np.float64) @ S.astype(np.float64).T
+    assert np.array_equal(e.rp_bwd(Xr, R, mode="bf16_signs"), (exact_b.astype(F32) * c).astype(F32))
+    # the general path on the same integers with an integer matrix: exact as well
+    Ri = rng.integers(-5, 6, (D, k)).astype(F32)
+    assert np.array_equal(e.rp_fwd(X, Ri, mode="bf16_split"), (X.astype(np.float64) @ Ri.astype(np.float64)).astype(F32))
+    assert np.array_equal(e.rp_bwd(Xr, Ri, mode="bf16_split"), (Xr.astype(np.float64) @ Ri.astype(np.float64).T).astype(F32))
+
+
+@pytest.mark.parametrize("mode", ["fp32", "bf16_split", "bf16_signs"])
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
 @pytest.mark.parametrize("supplied", [True, False])
 @pytest.mark.parametrize("N,D,frac", [(1, 256, 0.125), (31, 256, 0.125), (200, 256, 0.125), (130, 602, 0.125),
                                       (140, 100, 0.25), (129, 256, 0.25), (64, 128, 0.5), (77, 50, 0.3), (130, 7, 0.5),
                                       (100, 256, 0.49), (261, 602, 0.2)])
-def test_projection_and_quantisation_in_one_launch_equal_the_two_launches(N, D, frac, bits, supplied):
+def test_projection_and_quantisation_in_one_launch_equal_the_two_launches(N, D, frac, bits, supplied, mode):
     """exact_rp_minmax_pack_f32 == exact_rp_fwd_f32 followed by the oracle's
     quantize_activation of that product, bit for bit (packed bytes, fp32 and
     bf16 scale / min), with supplied noise and with the internal Philox stream."""
     k = o.kept_acts(frac, D)
     rng = np.random.default_rng(N * 7 + D + bits)
-    R = o.gaussian_matrix(D, k, rng)
+    R = o.rademacher_matrix(D, k, rng) if mode == "bf16_signs" else o.gaussian_matrix(D, k, rng)
     X = rng.standard_normal((N, D)).astype(F32)
     if N > 4:
         X[3] = 0.0                                  # a constant (all-zero) projected row: scale = inf
-    reduced = e.rp_fwd(X, R)
+    reduced = e.rp_fwd(X, R, mode=mode)
     noise = rng.random((N, k), dtype=F32) if supplied else o.philox_noise_rows(91, 4 * bits, N, k)
     want_packed, _, want_sbf, want_mbf, want_scale, want_mn = o.quantize_activation(reduced, bits, noise)
-    packed, s32, m32, sbf, mbf = e.rp_minmax_pack(X, R, bits, noise if supplied else None, 91, 4 * bits)
+    packed, s32, m32, sbf, mbf = e.rp_minmax_pack(X, R, bits, noise if supplied else None, 91, 4 * bits, mode=mode)
     assert np.array_equal(m32.view(np.uint32), want_mn.view(np.uint32))
     assert np.array_equal(s32.view(np.uint32), want_scale.view(np.uint32))
     assert np.array_equal(sbf, want_sbf) and np.array_equal(mbf, want_mbf)

@@ -92,19 +92,24 @@ def test_column_sums_wider_than_256_through_the_c_abi(cuda, N, K):
     assert torch.equal(out[:K], x.double().sum(0).float()) and (out[K:] == -77.0).all()
 
 
+@pytest.mark.parametrize("path", ["fp32", "split", "signs"])
 @pytest.mark.parametrize("N,k,D", [(169343, 32, 256), (232965, 76, 602), (232965, 32, 256), (2449029, 25, 100),
                                    (2449029, 64, 256)])
-def test_rp2input_at_benchmark_size(cuda, N, k, D):
-    """rp2input (ops.py:121-125) = X_r . R^T through exact_rp_bwd_f32 at the
-    shapes of the three configurations: every element within 1e-5 of a float64
-    product, and sampled rows against the oracle's own routine."""
+def test_rp2input_at_benchmark_size(cuda, N, k, D, path):
+    """rp2input (ops.py:121-125) = X_r . R^T through exact_rp_bwd_f32 /
+    exact_rp_bwd_bf16_f32 at the shapes of the three configurations, on every
+    matrix-core path: every element within 1e-5 of a float64 product, and
+    sampled rows against the oracle's own routine."""
     from exact_amd import ops
-    print(f"case rp2input N={N} k={k} D={D}", flush=True)
+    print(f"case rp2input N={N} k={k} D={D} {path}", flush=True)
     rng = np.random.default_rng(N + k)
     R = o.rademacher_matrix(D, k, rng)
     g = torch.Generator(device=cuda).manual_seed(N + D)
     xr = torch.randn(N, k, generator=g, device=cuda)
     r = dev(R)
+    config.rp_matrix_cores = "fp32" if path == "fp32" else "bf16"
+    if path == "signs":
+        r._exact_sign_matrix = True
     got = ops.rp2input(xr, (N, D), r)
     assert got.shape == (N, D)
     want = xr.double() @ r.double().t()

@@ -76,8 +76,14 @@ def test_the_one_launch_form_is_used_and_has_its_limits(backend, monkeypatch):
     A = sp.random(50, 50, 0.1, format="csr", random_state=1, dtype="float32")
     adj = SparseTensor.from_scipy(A, backend).set_value(None)
     conv = exact.QSAGEConv(64, 8).to(backend).train()
+    config.sage_aggregate_projected = False
     conv(x.detach().requires_grad_(), adj).sum().backward()
     assert len(calls) == 3
+    # aggregating the projected input (k + out = 24 < 64 columns): lin_l's copy is the quantised aggregate of x R,
+    # so only the shared copy goes through the one-launch form
+    config.sage_aggregate_projected = True
+    conv(x.detach().requires_grad_(), adj).sum().backward()
+    assert len(calls) == 4
     # the scheme's use counter still ticks
     class Scheme:
         n = 0
