@@ -144,7 +144,7 @@ class QSAGEConv(SAGEConv):
         2-D input for both sides, root weight, sum or mean aggregation, edge
         values without a gradient), else None."""
         if not (config.sage_single_node and self.training and self.root_weight and x.dim() == 2
-                and x.dtype == torch.float32 and not torch.is_autocast_enabled()
+                and x.dtype == torch.float32 and not torch.is_autocast_enabled(x.device.type)
                 and self.msg_and_aggr_func.reduce in ("sum", "mean")):
             return None
         rowptr, col, value = adj_t.csr()
