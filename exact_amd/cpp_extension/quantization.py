@@ -178,15 +178,15 @@ RP_FP32, RP_BF16_SPLIT, RP_BF16_SIGNS = 0, 1, 2      # EXACT_RP_* of the C heade
 
 def rp_mode(rand_matrix):
     """Which matrix-core path multiplies by this projection matrix.
-    config.rp_matrix_cores == "fp32": the fp32 instruction.  "bf16" (default):
+    config.matrix_cores == "fp32": the fp32 instruction.  "bf16" (default):
     the bf16 instruction on operands split into three bf16 pieces each -- for a
     matrix that ops._projection_matrix drew as +-c (it marks the tensor) on its
     signs alone, scaled by c at the end; for any other matrix the general
     six-product form."""
-    if config.rp_matrix_cores == "fp32":
+    if config.matrix_cores == "fp32":
         return RP_FP32
-    if config.rp_matrix_cores != "bf16":
-        raise ValueError("config.rp_matrix_cores must be 'bf16' or 'fp32'")
+    if config.matrix_cores != "bf16":
+        raise ValueError("config.matrix_cores must be 'bf16' or 'fp32'")
     return RP_BF16_SIGNS if getattr(rand_matrix, "_exact_sign_matrix", False) else RP_BF16_SPLIT
 
 

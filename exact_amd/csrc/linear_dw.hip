@@ -25,11 +25,9 @@
 // MFMA 32x32x2 f32 accumulator layout (wave64): register v of lane l is
 // C[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
 
-#include "exact_common.hpp"
+#include "bf16_split.hpp"
 
 namespace exact {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kDwPairs = 4;  // row pairs per batch of loads
 
@@ -124,7 +122,116 @@ __global__ __launch_bounds__(kBlock) void linear_dw_kernel(const float* __restri
     }
 }
 
+// The same product on the bf16 matrix cores at fp32 accuracy (bf16_split.hpp):
+// v_mfma_f32_32x32x16_bf16 reduces over 16 rows per instruction, lane (column,
+// g) holding rows n + 8 g .. n + 8 g + 7 of its column -- eight 4-byte loads
+// per operand fragment, each again 128 consecutive bytes per half-wave.  Both
+// operands are split into three bf16 pieces in registers and every 32 x 32
+// block takes six instructions per 16 rows, 3 / 8 of the matrix-core time of
+// the fp32 instruction.
 template <int MK, int MD, int WK>
+__global__ __launch_bounds__(kBlock, 2) void linear_dw_bf16_kernel(const float* __restrict__ dY, int64_t ldy,
+                                                                const float* __restrict__ X, int64_t ldx, int64_t N,
+                                                                int Kout, int D, int64_t rows_per_slab, int blocks_d,
+                                                                float* __restrict__ out) {
+  constexpr int WD = 4 / WK;
+  constexpr int64_t kRows = 16;  // rows per step
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int half = lane >> 5;
+  const int l32 = lane & 31;
+  const int bk = blockIdx.x / blocks_d, bd = blockIdx.x % blocks_d;
+  const int k0 = (bk * WK + wave / WD) * (32 * MK);
+  const int d0 = (bd * WD + wave % WD) * (32 * MD);
+  if (k0 >= Kout || d0 >= D) return;  // whole wavefront: no barrier follows
+  const int64_t n_begin = static_cast<int64_t>(blockIdx.y) * rows_per_slab;
+  const int64_t n_end = (n_begin + rows_per_slab < N) ? n_begin + rows_per_slab : N;
+
+  int kcol[MK], dcol[MD];
+#pragma unroll
+  for (int i = 0; i < MK; ++i) kcol[i] = min(k0 + 32 * i + l32, Kout - 1);
+#pragma unroll
+  for (int j = 0; j < MD; ++j) dcol[j] = min(d0 + 32 * j + l32, D - 1);
+
+  floatx16 acc[MK][MD];
+#pragma unroll
+  for (int i = 0; i < MK; ++i)
+#pragma unroll
+    for (int j = 0; j < MD; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const float* ycol[MK];
+  const float* xcol[MD];
+#pragma unroll
+  for (int i = 0; i < MK; ++i) ycol[i] = dY + kcol[i];
+#pragma unroll
+  for (int j = 0; j < MD; ++j) xcol[j] = X + dcol[j];
+  auto load_step = [&](int64_t n0, float (&a)[MK][8], float (&b)[MD][8]) {
+    if (n0 + kRows <= n_end) {  // wave-uniform: the whole step lies inside the slab, nothing to clamp or mask
+      const int64_t first = n0 + 8 * half;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+#pragma unroll
+        for (int i = 0; i < MK; ++i) a[i][e] = ycol[i][(first + e) * ldy];
+#pragma unroll
+        for (int j = 0; j < MD; ++j) b[j][e] = xcol[j][(first + e) * ldx];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int64_t row = n0 + 8 * half + e;
+        const int64_t rc = row < N ? row : N - 1;
+        const bool ok = row < n_end;
+#pragma unroll
+        for (int i = 0; i < MK; ++i) {
+          const float v = ycol[i][rc * ldy];
+          a[i][e] = ok ? v : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < MD; ++j) {
+          const float v = xcol[j][rc * ldx];
+          b[j][e] = ok ? v : 0.f;
+        }
+      }
+    }
+  };
+  // One set of raw registers: a step's values are split into their bf16 pieces first, then the
+  // loads of the next step are issued into the same registers and fly during this step's MFMAs.
+  float a[MK][8], b[MD][8];
+  int64_t n0 = n_begin;
+  if (n0 < n_end) load_step(n0, a, b);
+  while (n0 < n_end) {
+    Split8 sa[MK], sb[MD];
+#pragma unroll
+    for (int i = 0; i < MK; ++i) sa[i] = split3x8(a[i]);
+#pragma unroll
+    for (int j = 0; j < MD; ++j) sb[j] = split3x8(b[j]);
+    load_step(n0 + kRows, a, b);  // past the slab: clamped addresses, zeroed values
+#pragma unroll
+    for (int i = 0; i < MK; ++i)
+#pragma unroll
+      for (int j = 0; j < MD; ++j) {
+        const u32x4 pieces[3] = {sb[j].hi, sb[j].mid, sb[j].lo};
+        acc[i][j] = step_product<3>(sa[i], pieces, acc[i][j]);
+      }
+    n0 += kRows;
+  }
+
+#pragma unroll
+  for (int i = 0; i < MK; ++i)
+#pragma unroll
+    for (int j = 0; j < MD; ++j) {
+      const int cj = d0 + 32 * j + l32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ri = k0 + 32 * i + 8 * (v / 4) + 4 * half + (v % 4);
+        if (ri < Kout && cj < D) unsafeAtomicAdd(out + static_cast<int64_t>(ri) * D + cj, acc[i][j][v]);
+      }
+    }
+}
+
+template <int MK, int MD, int WK, bool BF16>
 static void launch_dw(const float* dY, int64_t ldy, const float* X, int64_t ldx, int64_t N, int Kout, int D, float* out,
                       hipStream_t s) {
   constexpr int WD = 4 / WK;
@@ -135,10 +242,39 @@ static void launch_dw(const float* dY, int64_t ldy, const float* X, int64_t ldx,
   int64_t slabs = (1024 + blocks - 1) / blocks;
   int64_t rows = (N + slabs - 1) / slabs;
   if (rows < 512) rows = 512;
-  rows = (rows + 2 * kDwPairs - 1) / (2 * kDwPairs) * (2 * kDwPairs);
+  rows = (rows + 15) / 16 * 16;  // whole batches (8 rows) resp. steps (16 rows)
   slabs = (N + rows - 1) / rows;
-  hipLaunchKernelGGL((linear_dw_kernel<MK, MD, WK>), dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(slabs)),
-                     dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, out);
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(slabs));
+  if (BF16) hipLaunchKernelGGL((linear_dw_bf16_kernel<MK, MD, WK>), grid, dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, out);
+  else hipLaunchKernelGGL((linear_dw_kernel<MK, MD, WK>), grid, dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, out);
+}
+
+template <bool BF16>
+static int linear_dw_any(const float* dY, int64_t ldy, const float* X, int64_t ldx, int64_t N, int64_t Kout, int64_t D,
+                         float* out, hipStream_t s) {
+  if (N < 0 || Kout < 0 || D < 0 || Kout > 65536 || D > 65536 || N > (int64_t{1} << 40)) return EXACT_E_SHAPE;
+  if (ldy < Kout || ldx < D) return EXACT_E_SHAPE;
+  if (Kout == 0 || D == 0) return EXACT_OK;
+  if (!out || (N > 0 && (!dY || !X))) return EXACT_E_NULL;
+  const int64_t total = Kout * D;
+  hipLaunchKernelGGL(dw_zero_kernel, dim3(static_cast<unsigned>((total + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, out, total);
+  if (N > 0) {
+    const int K = static_cast<int>(Kout), Dd = static_cast<int>(D);
+    // wavefront block: up to 64 x 64 of dW (wider blocks need more accumulator registers than two wavefronts
+    // per SIMD leave); the four wavefronts side by side along the longer extent when the other fits one wavefront
+    if (K <= 32) {
+      if (Dd <= 128) launch_dw<1, 1, 1, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+      else launch_dw<1, 2, 1, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+    } else if (K <= 64) {
+      if (Dd <= 128) launch_dw<2, 1, 1, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+      else launch_dw<2, 2, 1, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+    } else {
+      if (Dd <= 32) launch_dw<2, 1, 4, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+      else if (Dd <= 64) launch_dw<2, 2, 4, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+      else launch_dw<2, 2, 2, BF16>(dY, ldy, X, ldx, N, K, Dd, out, s);
+    }
+  }
+  return launch_status();
 }
 
 }  // namespace exact
@@ -149,30 +285,12 @@ extern "C" {
 
 int exact_linear_dw_f32(const float* dY, int64_t ldy, const float* X, int64_t ldx, int64_t N, int64_t Kout, int64_t D,
                         float* out, void* stream) {
-  if (N < 0 || Kout < 0 || D < 0 || Kout > 65536 || D > 65536 || N > (int64_t{1} << 40)) return EXACT_E_SHAPE;
-  if (ldy < Kout || ldx < D) return EXACT_E_SHAPE;
-  if (Kout == 0 || D == 0) return EXACT_OK;
-  if (!out || (N > 0 && (!dY || !X))) return EXACT_E_NULL;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t total = Kout * D;
-  hipLaunchKernelGGL(dw_zero_kernel, dim3(static_cast<unsigned>((total + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, out, total);
-  if (N > 0) {
-    const int K = static_cast<int>(Kout), Dd = static_cast<int>(D);
-    // wavefront block: up to 64 x 64 of dW (wider blocks need more accumulator registers than two wavefronts
-    // per SIMD leave); the four wavefronts side by side along the longer extent when the other fits one wavefront
-    if (K <= 32) {
-      if (Dd <= 128) launch_dw<1, 1, 1>(dY, ldy, X, ldx, N, K, Dd, out, s);
-      else launch_dw<1, 2, 1>(dY, ldy, X, ldx, N, K, Dd, out, s);
-    } else if (K <= 64) {
-      if (Dd <= 128) launch_dw<2, 1, 1>(dY, ldy, X, ldx, N, K, Dd, out, s);
-      else launch_dw<2, 2, 1>(dY, ldy, X, ldx, N, K, Dd, out, s);
-    } else {
-      if (Dd <= 32) launch_dw<2, 1, 4>(dY, ldy, X, ldx, N, K, Dd, out, s);
-      else if (Dd <= 64) launch_dw<2, 2, 4>(dY, ldy, X, ldx, N, K, Dd, out, s);
-      else launch_dw<2, 2, 2>(dY, ldy, X, ldx, N, K, Dd, out, s);
-    }
-  }
-  return launch_status();
+  return linear_dw_any<false>(dY, ldy, X, ldx, N, Kout, D, out, static_cast<hipStream_t>(stream));
+}
+
+int exact_linear_dw_bf16_f32(const float* dY, int64_t ldy, const float* X, int64_t ldx, int64_t N, int64_t Kout, int64_t D,
+                             float* out, void* stream) {
+  return linear_dw_any<true>(dY, ldy, X, ldx, N, Kout, D, out, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -36,79 +36,13 @@
 // (col, h) holding R[32 tile + col][16 step + 8 h + i].  SIGNS: one piece (the
 // signs as +-1 in bf16); SPLIT: three (hi, mid, lo).  Padding entries are 0.
 
+#include "bf16_split.hpp"
 #include "rp_common.hpp"
 
 namespace exact {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
 constexpr int kStepFeatures = 16;  // K of one MFMA
 constexpr int kSplitWaves = 4;     // wavefronts of a workgroup that share one 32-row tile
-
-// two fp32 -> two bf16 (round to nearest even) in one 32-bit word, `a` in the low half
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  const floatx2 f = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
-}
-__device__ __forceinline__ float low_bf16(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float high_bf16(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
-
-// error-free split of a pair of fp32 numbers into three bf16 pairs
-__device__ __forceinline__ void split3(float a, float b, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
-  hi = pack_bf16x2(a, b);
-  const float ra = a - low_bf16(hi), rb = b - high_bf16(hi);
-  mid = pack_bf16x2(ra, rb);
-  lo = pack_bf16x2(ra - low_bf16(mid), rb - high_bf16(mid));
-}
-
-struct Split8 {
-  u32x4 hi, mid, lo;
-};
-__device__ __forceinline__ Split8 split3x8(const float (&v)[8]) {
-  Split8 s;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    uint32_t h, m, l;
-    split3(v[2 * i], v[2 * i + 1], h, m, l);
-    s.hi[i] = h;
-    s.mid[i] = m;
-    s.lo[i] = l;
-  }
-  return s;
-}
-
-__device__ __forceinline__ floatx16 mfma_bf16(u32x4 a, u32x4 b, floatx16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0,
-                                                 0);
-}
-
-// +-1 (or 0 for a padding entry) as bf16 bits
-__device__ __forceinline__ uint32_t sign_bf16(float r, bool inside) {
-  return inside ? (0x3F80u | ((__float_as_uint(r) >> 16) & 0x8000u)) : 0u;
-}
-
-// acc += A-pieces . B-pieces for one k-step and one column tile.  BP == 1: B is a
-// sign matrix (one fragment); BP == 3: B split in three (hi, mid, lo), six products,
-// the small ones first.
-template <int BP>
-__device__ __forceinline__ floatx16 step_product(const Split8& a, const u32x4* b, floatx16 c) {
-  if constexpr (BP == 1) {
-    c = mfma_bf16(a.lo, b[0], c);
-    c = mfma_bf16(a.mid, b[0], c);
-    c = mfma_bf16(a.hi, b[0], c);
-  } else {
-    c = mfma_bf16(a.mid, b[1], c);
-    c = mfma_bf16(a.lo, b[0], c);
-    c = mfma_bf16(a.hi, b[2], c);
-    c = mfma_bf16(a.mid, b[0], c);
-    c = mfma_bf16(a.hi, b[1], c);
-    c = mfma_bf16(a.hi, b[0], c);
-  }
-  return c;
-}
 
 // Eight consecutive floats of a row starting at column `col`, zeros from column
 // `limit` on; VEC = the widest aligned access (limit % VEC == 0, col % VEC == 0).

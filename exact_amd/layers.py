@@ -16,7 +16,7 @@ from .conf import config
 from .cpp_extension import quantization as ext_quantization
 from .nn import GCN2Conv, GCNConv, GENConv, GraphConv, SAGEConv, glorot
 from .ops import (CompressedActivation, bn_relu_dropout, consumer_bits, project_and_quantize, qbatch_norm, qelu,
-                  qlinear, qsage, quantize_activation, relu_dropout, take_compressed)
+                  qgcn, qlinear, qsage, quantize_activation, relu_dropout, take_compressed)
 from .qsheme import QScheme
 from .spmm import QMatmul, qmatmul
 
@@ -100,8 +100,33 @@ class QGCNConv(GCNConv):
         # qlinear without a scheme.  Here the scheme is passed as scheme.
         return qlinear.apply(x, self.weight, None, take_compressed(x), None, self.lin_scheme)
 
+    def _as_one_node(self, x, adj_t):
+        """The whole layer through ops.qgcn where that node applies (fp32 2-D
+        input, sum or mean aggregation, edge values without a gradient), else
+        None."""
+        reduce = self.msg_and_aggr_func.reduce
+        if not (config.gcn_single_node and self.training and x.dim() == 2 and x.dtype == torch.float32
+                and not torch.is_autocast_enabled(x.device.type) and reduce in ("sum", "mean")):
+            return None
+        rowptr, col, value = adj_t.csr()
+        if value is not None and (value.requires_grad or value.dtype != torch.float32):
+            return None
+        st = adj_t.storage
+        # the transpose operands: backward multiplies by A^T (the reference builds them whenever the dense operand
+        # of its qspmm needs a gradient, spmm.py:34-44, which x W^T always does)
+        graph = (st.row(), rowptr, col, value, st.rowcount(), st.colptr(), st.csr2csc())
+        quantized = take_compressed(x)               # a copy a fused producer made, if any
+        if quantized is not None:
+            kept = CompressedActivation.adopt(x, quantized, None)
+        else:
+            kept = CompressedActivation.compress(x, self.lin_scheme)
+        return qgcn.apply(x, self.weight, self.bias, graph, reduce, kept)
+
     def forward(self, x, edge_index, edge_weight=None):
         adj_t = self._normalized(edge_index)
+        out = self._as_one_node(x, adj_t)
+        if out is not None:
+            return out
         out = self.message_and_aggregate(adj_t, self._transform(x))
         return out if self.bias is None else out + self.bias
 

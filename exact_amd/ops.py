@@ -499,6 +499,75 @@ class qsage(Function):
         return grad_x, grad_wl, grad_b, grad_wr, None, None, None, None
 
 
+class qgcn(Function):
+    """`aggregate(x W^T) + b` of a GCN layer as ONE autograd node: the chain
+    qlinear -> qspmm_sum -> bias add of the reference's QGCNConv.forward
+    (layers.py:244-262), keeping exactly what that chain keeps for backward
+    (the compressed copy of x that serves the weight gradient) and returning
+    the same gradients.  Aggregation and the linear map commute,
+    A (X W^T) = (A X) W^T, so the node runs the sparse product on the narrower
+    side (config.gcn_aggregate_narrow):
+
+      forward   in < out: (A X) W^T + b, the bias folded into the GEMM;
+                otherwise A (X W^T) + b as in the reference.
+      backward  G = A^T dY serves both dX = G W and dW = G^T X_hat.  Where dX is
+                not wanted (the first layer) and the kept copy is narrower
+                than `out`, dW = dY^T (A X_hat) instead: the sparse product
+                runs on the restored (still projected) copy.
+
+    Same numbers up to the order of fp32 sums.  `graph` = (row, rowptr, col,
+    value, rowcount, colptr, csr2csc) without a gradient for `value`; `kept` =
+    the CompressedActivation of x."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, graph, reduce, kept):
+        row, rowptr, col, value, rowcount, colptr, csr2csc = graph
+        cout, cin = weight.shape
+        if config.gcn_aggregate_narrow and cin < cout:
+            aggregated = spmm.spmm_csr(rowptr, col, value, x, reduce)
+            out = aggregated.mm(weight.t()) if bias is None else torch.addmm(bias, aggregated, weight.t())
+            del aggregated
+        else:
+            out = spmm.spmm_csr(rowptr, col, value, x.mm(weight.t()), reduce)
+            if bias is not None:
+                out += bias
+        empty_cache(config.empty_cache_threshold)
+        ctx.kept, ctx.weight, ctx.has_bias = kept, weight, bias is not None
+        ctx.graph, ctx.reduce = graph, reduce
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        row, rowptr, col, value, rowcount, colptr, csr2csc = ctx.graph
+        weight = ctx.weight
+        kept, ctx.kept = ctx.kept, None
+        grad_output = grad_output.contiguous()
+        has_value = value is not None
+        cout = weight.shape[0]
+        grad_x = grad_w = None
+        stored_width = kept.stored_shape[1]
+        if not ctx.needs_input_grad[0] and ctx.needs_input_grad[1] and config.gcn_aggregate_narrow and stored_width < cout:
+            # dW = dY^T (A X_hat); with a projection X_hat = X_r R^T and the sparse product runs on X_r
+            x_r = dequantize_activation(kept.quantized, kept.stored_shape)
+            grad_w = ext_backward_func.weight_gradient(grad_output, spmm.spmm_csr(rowptr, col, value, x_r, ctx.reduce))
+            if kept.randmat is not None:
+                grad_w = grad_w.mm(kept.randmat.t())
+        else:
+            if ctx.reduce == "sum":
+                g = spmm.spmm_sum_bw(row, rowptr, col, value, colptr, csr2csc, None, grad_output, has_value, False, True)[1]
+            else:
+                g = spmm.spmm_mean_bw(row, rowptr, col, value, rowcount, colptr, csr2csc, None, grad_output, has_value,
+                                      False, True)[1]
+            if ctx.needs_input_grad[0]:
+                grad_x = g.mm(weight)
+            if ctx.needs_input_grad[1]:
+                grad_w = _restored_weight_gradient(g, kept)
+        del kept
+        grad_b = ext_backward_func.column_sums(grad_output) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        empty_cache(config.empty_cache_threshold)
+        return grad_x, grad_w, grad_b, None, None, None
+
+
 class qelu(Function):
     """ELU that keeps its input compressed (reference ops.py:182-204)."""
 

@@ -225,6 +225,11 @@ int exact_stream_probe_f32(const float *x, int64_t n, int out_bytes, void *out, 
  * is cut into slabs combined by fp32 atomics: the summation order is not fixed. */
 int exact_linear_dw_f32(const float *dY, int64_t ldy, const float *X, int64_t ldx, int64_t N,
                         int64_t Kout, int64_t D, float *out, void *stream);
+/* The same product on the bf16 matrix cores at fp32 accuracy: both operands are split, without error, into three
+ * bf16 pieces and six bf16 products replace each fp32 product (the neglected ones are below 2^-24 of it).  Same
+ * arguments and limits; results agree with exact_linear_dw_f32 to fp32 rounding. */
+int exact_linear_dw_bf16_f32(const float *dY, int64_t ldy, const float *X, int64_t ldx, int64_t N,
+                             int64_t Kout, int64_t D, float *out, void *stream);
 
 /* Fused epilogues (no single counterpart in the reference: each replaces a
  * chain of its calls with one pass over the data, bit-identical to the chain).

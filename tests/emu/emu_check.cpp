@@ -511,15 +511,18 @@ static void check_dw(int64_t N, int64_t K, int64_t D, int64_t pad, std::mt19937&
   Buf<float> dy(static_cast<size_t>(N * ldy)), x(static_cast<size_t>(N * ldx)), out(static_cast<size_t>(K * D));
   for (int64_t i = 0; i < N * ldy; ++i) dy[i] = static_cast<float>(id(rng));
   for (int64_t i = 0; i < N * ldx; ++i) x[i] = static_cast<float>(id(rng));
-  const int rc = exact_linear_dw_f32(dy.p, ldy, x.p, ldx, N, K, D, out.p, nullptr);
-  CHECK(rc == 0, "dw rc %d", rc);
-  for (int64_t k = 0; k < K; ++k)
-    for (int64_t d = 0; d < D; ++d) {
-      double want = 0;
-      for (int64_t n = 0; n < N; ++n) want += static_cast<double>(dy[n * ldy + k]) * x[n * ldx + d];
-      CHECK(out[k * D + d] == static_cast<float>(want), "dw N=%lld K=%lld D=%lld at (%lld, %lld)", (long long)N,
-            (long long)K, (long long)D, (long long)k, (long long)d);
-    }
+  for (int bf16 = 0; bf16 < 2; ++bf16) {  // the fp32 and the bf16 matrix-core kernel
+    const int rc = bf16 ? exact_linear_dw_bf16_f32(dy.p, ldy, x.p, ldx, N, K, D, out.p, nullptr)
+                        : exact_linear_dw_f32(dy.p, ldy, x.p, ldx, N, K, D, out.p, nullptr);
+    CHECK(rc == 0, "dw rc %d", rc);
+    for (int64_t k = 0; k < K; ++k)
+      for (int64_t d = 0; d < D; ++d) {
+        double want = 0;
+        for (int64_t n = 0; n < N; ++n) want += static_cast<double>(dy[n * ldy + k]) * x[n * ldx + d];
+        CHECK(out[k * D + d] == static_cast<float>(want), "dw bf16=%d N=%lld K=%lld D=%lld at (%lld, %lld)", bf16, (long long)N,
+              (long long)K, (long long)D, (long long)k, (long long)d);
+      }
+  }
 }
 
 static const int64_t kRpShapes[][3] = {{1, 256, 32}, {31, 256, 32}, {200, 256, 32}, {130, 602, 76}, {140, 100, 25}, {129, 256, 64},
@@ -534,6 +537,18 @@ int main(int argc, char** argv) {
   if (mode == "rp") {  // the projection kernels only
     for (auto& s : kRpShapes) check_rp(s[0], s[1], s[2], rng);
     std::printf("rp shapes ok (failures so far %d)\n", g_fail);
+    return g_fail != 0;
+  }
+  if (mode == "dw") {  // the weight-gradient kernels only
+    check_dw(1, 1, 1, 0, rng);
+    check_dw(7, 3, 5, 2, rng);
+    check_dw(100, 40, 256, 0, rng);
+    check_dw(515, 256, 128, 3, rng);
+    check_dw(333, 47, 25, 1, rng);
+    check_dw(600, 130, 70, 0, rng);
+    check_dw(513, 32, 200, 5, rng);
+    check_dw(1100, 256, 256, 0, rng);
+    std::printf("dw shapes ok (failures so far %d)\n", g_fail);
     return g_fail != 0;
   }
   const int64_t shapes[][2] = {{1, 1}, {5, 3}, {37, 25}, {64, 32}, {100, 76}, {33, 40}, {129, 100}, {300, 128},

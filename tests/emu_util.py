@@ -448,8 +448,8 @@ def col_moments(x, center, guard=8, expect_rc=0):
     return a[:K], b[:K]
 
 
-def linear_dw(dy, x, ldy=None, ldx=None, guard=8, expect_rc=0):
-    """exact_linear_dw_f32 -> fp32 [Kout, D]; dy / x may be given wider than used (row strides)."""
+def linear_dw(dy, x, ldy=None, ldx=None, guard=8, expect_rc=0, bf16=False):
+    """exact_linear_dw_f32 / exact_linear_dw_bf16_f32 -> fp32 [Kout, D]; dy / x may be given wider than used (row strides)."""
     dy, x = f32(dy), f32(x)
     N, K = dy.shape
     D = x.shape[1]
@@ -458,7 +458,8 @@ def linear_dw(dy, x, ldy=None, ldx=None, guard=8, expect_rc=0):
     if ldx:
         wide = np.full((N, ldx), np.float32(np.nan), np.float32); wide[:, :D] = x; x = wide
     out = np.full(K * D + guard, np.float32(-777.0), np.float32)
-    rc = emu().exact_linear_dw_f32(p(dy), dy.shape[1], p(x), x.shape[1], N, K, D, p(out), None)
+    fn = emu().exact_linear_dw_bf16_f32 if bf16 else emu().exact_linear_dw_f32
+    rc = fn(p(dy), dy.shape[1], p(x), x.shape[1], N, K, D, p(out), None)
     assert rc == expect_rc, rc
     if rc:
         return None

@@ -35,15 +35,17 @@ DW_SHAPES = [(256, 256), (256, 128), (40, 256), (256, 64), (47, 64), (256, 25), 
              (16, 64), (24, 300), (64, 256), (256, 32), (300, 64), (256, 602)]
 
 
+@pytest.mark.parametrize("cores", ["bf16", "fp32"])
 @pytest.mark.parametrize("N", BIG)
 @pytest.mark.parametrize("K,D", DW_SHAPES)
-def test_weight_gradient_is_the_integer_product_at_benchmark_size(cuda, N, K, D):
+def test_weight_gradient_is_the_integer_product_at_benchmark_size(cuda, N, K, D, cores):
     """exact_linear_dw_f32 on small integers: every product and every partial
     sum is an integer below 2^24, so fp32 is exact whatever the order and the
     result must equal the float64 product bit for bit -- a wrong fragment, a
     row counted twice or missed, or a lost atomic shows.  Contiguous and with
     row strides longer than the width (NaN in the padding)."""
-    print(f"case dW N={N} K={K} D={D}", flush=True)
+    print(f"case dW N={N} K={K} D={D} {cores}", flush=True)
+    config.matrix_cores = cores
     dy, x = _ints((N, K), cuda, N + K), _ints((N, D), cuda, N + D + 1)
     want = (dy.double().t() @ x.double()).float()
     got = bf.weight_gradient(dy, x)
@@ -54,14 +56,19 @@ def test_weight_gradient_is_the_integer_product_at_benchmark_size(cuda, N, K, D)
     assert torch.equal(bf.weight_gradient(wide_dy[:, 2:2 + K], wide_x[:, 5:5 + D]), want)
 
 
-@pytest.mark.parametrize("N,K,D", [(20000, 1024, 1024), (16384, 1000, 513), (50000, 1, 1), (30011, 7, 1024)])
-def test_weight_gradient_limits_of_the_wrapper(cuda, N, K, D):
-    """The widest operands the wrapper hands to the kernel, and the narrowest."""
-    print(f"case dW N={N} K={K} D={D}", flush=True)
+@pytest.mark.parametrize("cores", ["bf16", "fp32"])
+@pytest.mark.parametrize("N,K,D", [(20000, 1024, 1024), (16384, 1000, 513), (50000, 1, 1), (30011, 7, 1024), (169343, 256, 256)])
+def test_weight_gradient_limits_of_the_wrapper(cuda, N, K, D, cores):
+    """The widest operands the wrapper hands to the kernel, and the narrowest;
+    random operands with rows of very different size within 1e-5 of the sum of
+    the absolute terms."""
+    print(f"case dW N={N} K={K} D={D} {cores}", flush=True)
+    config.matrix_cores = cores
     dy, x = _ints((N, K), cuda, 1), _ints((N, D), cuda, 2)
     assert torch.equal(bf.weight_gradient(dy, x), (dy.double().t() @ x.double()).float())
     g = torch.Generator(device=cuda).manual_seed(3)
-    dy, x = torch.randn(N, K, generator=g, device=cuda), torch.randn(N, D, generator=g, device=cuda)
+    spread = torch.exp(8 * torch.rand(N, 1, generator=g, device=cuda) - 4)
+    dy, x = torch.randn(N, K, generator=g, device=cuda) * spread, torch.randn(N, D, generator=g, device=cuda) * spread
     want = dy.double().t() @ x.double()
     bound = dy.abs().double().t() @ x.abs().double()
     assert ((bf.weight_gradient(dy, x).double() - want).abs() <= 1e-5 * bound + 1e-30).all()
@@ -107,7 +114,7 @@ def test_rp2input_at_benchmark_size(cuda, N, k, D, path):
     g = torch.Generator(device=cuda).manual_seed(N + D)
     xr = torch.randn(N, k, generator=g, device=cuda)
     r = dev(R)
-    config.rp_matrix_cores = "fp32" if path == "fp32" else "bf16"
+    config.matrix_cores = "fp32" if path == "fp32" else "bf16"
     if path == "signs":
         r._exact_sign_matrix = True
     got = ops.rp2input(xr, (N, D), r)

@@ -20,10 +20,10 @@ def close(got, want, rtol=1e-5):
 
 
 def _matrix_on_device(R, path):
-    """The projection matrix as the given path wants it: config.rp_matrix_cores
+    """The projection matrix as the given path wants it: config.matrix_cores
     set, and for "signs" the mark that ops._projection_matrix puts on a +-c
     matrix it drew itself."""
-    config.rp_matrix_cores = "fp32" if path == "fp32" else "bf16"
+    config.matrix_cores = "fp32" if path == "fp32" else "bf16"
     r = dev(R)
     if path == "signs":
         assert (np.abs(R) == np.abs(R).max()).all()

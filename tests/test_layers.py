@@ -496,6 +496,91 @@ def test_sage_node_keeps_what_the_chain_keeps(backend):
     assert widths == [k + cout, cout]                  # forward at k + out = 44 instead of 96, backward at out = 20
 
 
+GCN_FORMS = {
+    "chain": dict(gcn_single_node=False),
+    "node": dict(gcn_single_node=True, gcn_aggregate_narrow=False),
+    "node+narrow": dict(gcn_single_node=True, gcn_aggregate_narrow=True),
+}
+
+
+@pytest.mark.parametrize("form", list(GCN_FORMS))
+@pytest.mark.parametrize("kept_frac,bits,cin,cout,x_grad", [(1.0, 8, 32, 72, False), (1.0, 8, 32, 72, True), (1.0, 8, 64, 24, True),
+                                                             (0.25, 8, 96, 40, False), (1.0, 2, 32, 72, False)])
+def test_gcn_layer_in_every_form_matches_the_oracle_chain(backend, form, kept_frac, bits, cin, cout, x_grad):
+    """QGCNConv (layers.py:244-262) as the reference's chain qlinear -> qspmm ->
+    bias and as one node with the sparse product on the narrower side of the
+    linear map (forward when in < out; backward, for a first layer, on the kept
+    copy), against the oracle's chain in the reference's order: output, input
+    gradient and bias gradient within 1e-5 of each tensor's largest entry; the
+    weight gradient passes through the kept, quantised copy and gets the
+    allowance of two codes that fall the other way (see the SAGE test)."""
+    config.kept_frac, config.activation_compression_bits = kept_frac, [bits]
+    for name, on in GCN_FORMS[form].items():
+        setattr(config, name, on)
+    n = 900
+    A = er_graph(n, 9, 6)
+    adj = gcn_norm(SparseTensor.from_scipy(A).set_value(None), add_self_loops=True)
+    rowptr, col, value = adj.csr()
+    graph = om.Graph(rowptr.numpy(), col.numpy(), value.numpy())
+    adj = adj.to(backend).fill_cache_()
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(n, cin, generator=g)
+    dy = torch.randn(n, cout, generator=g)
+    torch.manual_seed(6)
+    conv = exact.QGCNConv(cin, cout, normalize=False).to(backend).train()
+    with torch.no_grad():
+        conv.bias.copy_(torch.randn(cout, generator=g))
+    other = wire_noise(46)
+    xd = x.clone().to(backend).requires_grad_(x_grad)
+    y = conv(xd, adj)
+    y.backward(dy.to(backend))
+    mine = [y.detach().cpu(), xd.grad.cpu() if x_grad else None, conv.weight.grad.cpu(), conv.bias.grad.cpu()]
+    w, b = (p.detach().cpu().clone().requires_grad_() for p in (conv.weight, conv.bias))
+    xo = x.clone().requires_grad_(x_grad)
+    c = om.Ctx(bits, kept_frac, other.noise, other.rademacher)
+    yo = om.SpMMFn.apply(graph, om.QLinearFn.apply(c, xo, w, None, None, None, None), "sum") + b
+    yo.backward(dy)
+    want = [yo.detach(), xo.grad if x_grad else None, w.grad, b.grad]
+    k = ops.kept_columns(cin) if kept_frac < 1.0 else cin
+    r_max = k ** -0.5 if kept_frac < 1.0 else 1.0
+    step = 12.0 * (cin / k) ** 0.5 / (2 ** bits - 1)
+    g_max = 4.5 * 2.0                                   # |A^T dY| with sym-normalised rows (sums of weights stay below 2)
+    for name, a, bb in zip(("y", "dx", "dW", "db"), mine, want):
+        if a is None:
+            continue
+        scale = bb.abs().max().item()
+        err = (a - bb).abs().max().item()
+        allowed = 1e-5 * scale + (2 * step * g_max * r_max if name == "dW" else 0.0)
+        assert err <= allowed, (name, err, scale, allowed)
+
+
+def test_gcn_node_runs_the_sparse_product_on_the_narrow_side(backend):
+    from exact_amd.cpp_extension import spmm as ext_spmm
+    n, cin, cout = 500, 32, 72
+    adj = gcn_norm(SparseTensor.from_scipy(er_graph(n, 8, 2)).set_value(None), add_self_loops=True).to(backend).fill_cache_()
+    widths = []
+    real = ext_spmm.spmm_csr
+
+    def spy(rowptr, col, value, mat, reduce):
+        widths.append(mat.shape[1])
+        return real(rowptr, col, value, mat, reduce)
+
+    ext_spmm.spmm_csr = spy
+    try:
+        conv = exact.QGCNConv(cin, cout, normalize=False).to(backend).train()
+        conv(torch.randn(n, cin).to(backend), adj).sum().backward()               # a first layer: no input gradient
+        assert widths == [cin, cin]
+        del widths[:]
+        conv(torch.randn(n, cin).to(backend).requires_grad_(), adj).sum().backward()
+        assert widths == [cin, cout]
+        del widths[:]
+        narrowing = exact.QGCNConv(cout, cin, normalize=False).to(backend).train()
+        narrowing(torch.randn(n, cout).to(backend).requires_grad_(), adj).sum().backward()
+        assert widths == [cin, cin]
+    finally:
+        ext_spmm.spmm_csr = real
+
+
 def test_qmodule_conversion_and_state_dict(backend):
     net = GCN(16, 32, 4, 3, dropout=0.3, batch_norm=True)
     ref_keys = list(net.state_dict().keys())

@@ -674,9 +674,10 @@ def test_sparse_product_with_row_strides(backend):
     assert ext_spmm._aligned_rows(wide[:, 5:5 + K], A.nnz).data_ptr() == wide[:, 5:5 + K].data_ptr()
 
 
+@pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("N,K,D", [(1, 1, 1), (7, 3, 5), (100, 40, 256), (515, 256, 128), (1030, 64, 64), (333, 47, 25),
                                    (1201, 256, 76), (600, 130, 70), (513, 32, 200), (2100, 256, 256)])
-def test_weight_gradient_kernel(N, K, D):
+def test_weight_gradient_kernel(N, K, D, bf16):
     """exact_linear_dw_f32 = dY^T . X.  Small integers: every product and sum is
     exact in fp32, so the result must equal the integer GEMM bit for bit (a
     wrong fragment, a row counted twice or a column off by one shows); random
@@ -685,12 +686,15 @@ def test_weight_gradient_kernel(N, K, D):
     rng = np.random.default_rng(N + K + D)
     dy = rng.integers(-3, 4, (N, K)).astype(np.float32)
     x = rng.integers(-3, 4, (N, D)).astype(np.float32)
-    assert np.array_equal(e.linear_dw(dy, x), (dy.astype(np.float64).T @ x.astype(np.float64)).astype(np.float32))
-    assert np.array_equal(e.linear_dw(dy, x, ldy=K + 3, ldx=D + 9), (dy.astype(np.float64).T @ x.astype(np.float64)).astype(np.float32))
-    dy, x = rng.standard_normal((N, K)).astype(np.float32), rng.standard_normal((N, D)).astype(np.float32)
+    assert np.array_equal(e.linear_dw(dy, x, bf16=bf16), (dy.astype(np.float64).T @ x.astype(np.float64)).astype(np.float32))
+    assert np.array_equal(e.linear_dw(dy, x, ldy=K + 3, ldx=D + 9, bf16=bf16),
+                          (dy.astype(np.float64).T @ x.astype(np.float64)).astype(np.float32))
+    # rows of very different size: a dropped low-order piece of the bf16 form would show
+    dy = (rng.standard_normal((N, K)) * np.exp(rng.uniform(-4, 4, (N, 1)))).astype(np.float32)
+    x = (rng.standard_normal((N, D)) * np.exp(rng.uniform(-4, 4, (N, 1)))).astype(np.float32)
     want = dy.astype(np.float64).T @ x.astype(np.float64)
     bound = np.abs(dy).astype(np.float64).T @ np.abs(x).astype(np.float64)
-    assert (np.abs(e.linear_dw(dy, x) - want) <= 1e-5 * bound + 1e-30).all()
+    assert (np.abs(e.linear_dw(dy, x, bf16=bf16) - want) <= 1e-5 * bound + 1e-30).all()
 
 
 def test_weight_gradient_limits():
