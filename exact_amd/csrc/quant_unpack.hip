@@ -76,7 +76,14 @@ __device__ __forceinline__ void store_quad_half(half_t* __restrict__ p, int nv, 
 // reference's at::Half instantiation (at::Half operators evaluate in fp32 and
 // round to fp16), the quotient and the sum are each rounded to fp16
 // (quantization_cuda_kernel.cu:182).
-template <int BITS, int SLOTS, int VEC, int PARAM>
+//
+// ROWS consecutive rows per lane group.  A group issues every load of its rows
+// (packed words, scale, min) before the first value is used: with one row per
+// group a wavefront has a single 4-byte load in flight, and when the packed
+// stream comes from HBM rather than from L2 (backward reads what forward wrote
+// long before) the kernel runs at the speed of that latency -- measured 50 us
+// instead of 26 at [169343, 256].
+template <int BITS, int SLOTS, int VEC, int PARAM, int ROWS>
 __global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
   constexpr bool BF16P = PARAM == kParamBF16;
   constexpr bool F16 = PARAM == kParamF16;
@@ -86,68 +93,76 @@ __global__ __launch_bounds__(kBlock) void unpack_kernel(const UnpackArgs a) {
   const int lpr = 1 << a.lpr_log2;
   const int lane_in_row = t & (lpr - 1);
   const int rows_per_wg = kBlock >> a.lpr_log2;
-  const int64_t n = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (t >> a.lpr_log2);
-  if (n >= a.N) return;
+  const int64_t n_first = (static_cast<int64_t>(blockIdx.x) * rows_per_wg + (t >> a.lpr_log2)) * ROWS;
+  if (n_first >= a.N) return;
   const int quad_base = blockIdx.y * (lpr * SLOTS) + lane_in_row;
 
-  float sc, mnv;
-  if constexpr (BF16P) {
-    sc = bf16_to_f32(static_cast<const uint16_t*>(a.scale)[n]);
-    mnv = bf16_to_f32(static_cast<const uint16_t*>(a.mn)[n]);
-  } else if constexpr (F16) {
-    sc = static_cast<float>(static_cast<const half_t*>(a.scale)[n]);
-    mnv = static_cast<float>(static_cast<const half_t*>(a.mn)[n]);
-  } else {
-    sc = static_cast<const float*>(a.scale)[n];
-    mnv = static_cast<const float*>(a.mn)[n];
-  }
-  // One IEEE division per row instead of one per element: with rcp = RN(1/sc),
-  // exact_quotient() returns RN(q / sc) for every integer 0 <= q <= 255 as long
-  // as sc is a normal number far from the exponent limits; other rows divide.
-  const float asc = fabsf(sc);
-  const bool fast_div = asc >= 0x1p-64f && asc <= 0x1p64f;
-  const float rcp = 1.0f / sc;
-  const int shift = static_cast<int>(n & (WPT - 1)) * BITS;
-  const uint8_t* grp = a.packed + (n / WPT) * a.G;
-  float* orow = F16 ? nullptr : a.out + n * a.G;
-  half_t* orow_h = F16 ? reinterpret_cast<half_t*>(a.out) + n * a.G : nullptr;
-
-  uint32_t w[SLOTS];
+  float sc[ROWS], mnv[ROWS];
+  uint32_t w[ROWS][SLOTS];
 #pragma unroll
-  for (int s = 0; s < SLOTS; ++s) {
-    const int c = quad_base + s * lpr;
-    w[s] = 0;
-    if (c < a.qpr) {
-      if (a.in_vec == 4) {
-        w[s] = *reinterpret_cast<const uint32_t*>(grp + 4 * c);
-      } else {
-        const int cnt = min(4, a.G - 4 * c);
-        for (int i = 0; i < cnt; ++i) w[s] |= static_cast<uint32_t>(grp[4 * c + i]) << (8 * i);
-      }
-    }
-  }
-#pragma unroll
-  for (int s = 0; s < SLOTS; ++s) {
-    const int c = quad_base + s * lpr;
-    if (c >= a.qpr) continue;
-    const uint32_t f = (w[s] >> shift) & FIELD;
-    float r[4];
-    if (__builtin_expect(fast_div, 1)) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float quo = exact_quotient(static_cast<float>((f >> (8 * i)) & 0xFFu), sc, rcp);
-        r[i] = (F16 ? round_to_half(quo) : quo) + mnv;
-      }
+  for (int rr = 0; rr < ROWS; ++rr) {
+    const int64_t n = (n_first + rr < a.N) ? n_first + rr : a.N - 1;  // rows past the end repeat the last one; never stored
+    if constexpr (BF16P) {
+      sc[rr] = bf16_to_f32(static_cast<const uint16_t*>(a.scale)[n]);
+      mnv[rr] = bf16_to_f32(static_cast<const uint16_t*>(a.mn)[n]);
+    } else if constexpr (F16) {
+      sc[rr] = static_cast<float>(static_cast<const half_t*>(a.scale)[n]);
+      mnv[rr] = static_cast<float>(static_cast<const half_t*>(a.mn)[n]);
     } else {
+      sc[rr] = static_cast<const float*>(a.scale)[n];
+      mnv[rr] = static_cast<const float*>(a.mn)[n];
+    }
+    const uint8_t* grp = a.packed + (n / WPT) * a.G;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        // quantization_cuda_kernel.cu:182: true division, then add
-        const float quo = static_cast<float>((f >> (8 * i)) & 0xFFu) / sc;
-        r[i] = (F16 ? round_to_half(quo) : quo) + mnv;
+    for (int s = 0; s < SLOTS; ++s) {
+      const int c = quad_base + s * lpr;
+      w[rr][s] = 0;
+      if (c < a.qpr) {
+        if (a.in_vec == 4) {
+          w[rr][s] = *reinterpret_cast<const uint32_t*>(grp + 4 * c);
+        } else {
+          const int cnt = min(4, a.G - 4 * c);
+          for (int i = 0; i < cnt; ++i) w[rr][s] |= static_cast<uint32_t>(grp[4 * c + i]) << (8 * i);
+        }
       }
     }
-    if constexpr (F16) store_quad_half<VEC>(orow_h + 4 * c, min(4, a.G - 4 * c), r);  // rounds the sum to fp16
-    else store_quad<VEC>(orow + 4 * c, min(4, a.G - 4 * c), r);
+  }
+#pragma unroll
+  for (int rr = 0; rr < ROWS; ++rr) {
+    const int64_t n = n_first + rr;
+    if (n >= a.N) break;
+    // One IEEE division per row instead of one per element: with rcp = RN(1/sc),
+    // exact_quotient() returns RN(q / sc) for every integer 0 <= q <= 255 as long
+    // as sc is a normal number far from the exponent limits; other rows divide.
+    const float asc = fabsf(sc[rr]);
+    const bool fast_div = asc >= 0x1p-64f && asc <= 0x1p64f;
+    const float rcp = 1.0f / sc[rr];
+    const int shift = static_cast<int>(n & (WPT - 1)) * BITS;
+    float* orow = F16 ? nullptr : a.out + n * a.G;
+    half_t* orow_h = F16 ? reinterpret_cast<half_t*>(a.out) + n * a.G : nullptr;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      const int c = quad_base + s * lpr;
+      if (c >= a.qpr) continue;
+      const uint32_t f = (w[rr][s] >> shift) & FIELD;
+      float r[4];
+      if (__builtin_expect(fast_div, 1)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float quo = exact_quotient(static_cast<float>((f >> (8 * i)) & 0xFFu), sc[rr], rcp);
+          r[i] = (F16 ? round_to_half(quo) : quo) + mnv[rr];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // quantization_cuda_kernel.cu:182: true division, then add
+          const float quo = static_cast<float>((f >> (8 * i)) & 0xFFu) / sc[rr];
+          r[i] = (F16 ? round_to_half(quo) : quo) + mnv[rr];
+        }
+      }
+      if constexpr (F16) store_quad_half<VEC>(orow_h + 4 * c, min(4, a.G - 4 * c), r);  // rounds the sum to fp16
+      else store_quad<VEC>(orow + 4 * c, min(4, a.G - 4 * c), r);
+    }
   }
 }
 
@@ -180,20 +195,24 @@ static UnpackGeometry plan_unpack(int64_t G) {
 
 static bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-template <int BITS, int PARAM>
+template <int BITS, int PARAM, int ROWS>
 static void launch_unpack_variant(const UnpackArgs& a, int slots, bool vec4, dim3 grid, hipStream_t s) {
   if (slots == 1) {
     if (vec4)
-      hipLaunchKernelGGL((unpack_kernel<BITS, 1, 4, PARAM>), grid, dim3(kBlock), 0, s, a);
+      hipLaunchKernelGGL((unpack_kernel<BITS, 1, 4, PARAM, ROWS>), grid, dim3(kBlock), 0, s, a);
     else
-      hipLaunchKernelGGL((unpack_kernel<BITS, 1, 1, PARAM>), grid, dim3(kBlock), 0, s, a);
+      hipLaunchKernelGGL((unpack_kernel<BITS, 1, 1, PARAM, ROWS>), grid, dim3(kBlock), 0, s, a);
   } else {
     if (vec4)
-      hipLaunchKernelGGL((unpack_kernel<BITS, 2, 4, PARAM>), grid, dim3(kBlock), 0, s, a);
+      hipLaunchKernelGGL((unpack_kernel<BITS, 2, 4, PARAM, ROWS>), grid, dim3(kBlock), 0, s, a);
     else
-      hipLaunchKernelGGL((unpack_kernel<BITS, 2, 1, PARAM>), grid, dim3(kBlock), 0, s, a);
+      hipLaunchKernelGGL((unpack_kernel<BITS, 2, 1, PARAM, ROWS>), grid, dim3(kBlock), 0, s, a);
   }
 }
+
+// Rows per lane group: four once the launch has workgroups to spare (2048 at one row each, eight per compute
+// unit), one for small activations, where the number of wavefronts matters more than the loads each has in flight.
+constexpr int kUnpackRows = 4;
 
 template <int PARAM>
 static int unpack_common(const uint8_t* packed, int bits, const void* scale, const void* mn,
@@ -215,12 +234,24 @@ static int unpack_common(const uint8_t* packed, int bits, const void* scale, con
   a.in_vec = (G % 4 == 0 && aligned(packed, 4)) ? 4 : 1;
   const bool vec4 = (G % 4 == 0) && aligned(out, PARAM == kParamF16 ? 8 : 16);
   const int rows_per_wg = kBlock >> g.lpr_log2;
-  const dim3 grid(static_cast<unsigned>((N + rows_per_wg - 1) / rows_per_wg), static_cast<unsigned>(g.grid_y));
-  switch (bits) {
-    case 1: launch_unpack_variant<1, PARAM>(a, g.slots, vec4, grid, s); break;
-    case 2: launch_unpack_variant<2, PARAM>(a, g.slots, vec4, grid, s); break;
-    case 4: launch_unpack_variant<4, PARAM>(a, g.slots, vec4, grid, s); break;
-    default: launch_unpack_variant<8, PARAM>(a, g.slots, vec4, grid, s); break;
+  const int64_t wgs_one_row = (N + rows_per_wg - 1) / rows_per_wg;
+  if (wgs_one_row * g.grid_y >= 2048) {
+    const int64_t rows = static_cast<int64_t>(rows_per_wg) * kUnpackRows;
+    const dim3 grid(static_cast<unsigned>((N + rows - 1) / rows), static_cast<unsigned>(g.grid_y));
+    switch (bits) {
+      case 1: launch_unpack_variant<1, PARAM, kUnpackRows>(a, g.slots, vec4, grid, s); break;
+      case 2: launch_unpack_variant<2, PARAM, kUnpackRows>(a, g.slots, vec4, grid, s); break;
+      case 4: launch_unpack_variant<4, PARAM, kUnpackRows>(a, g.slots, vec4, grid, s); break;
+      default: launch_unpack_variant<8, PARAM, kUnpackRows>(a, g.slots, vec4, grid, s); break;
+    }
+  } else {
+    const dim3 grid(static_cast<unsigned>(wgs_one_row), static_cast<unsigned>(g.grid_y));
+    switch (bits) {
+      case 1: launch_unpack_variant<1, PARAM, 1>(a, g.slots, vec4, grid, s); break;
+      case 2: launch_unpack_variant<2, PARAM, 1>(a, g.slots, vec4, grid, s); break;
+      case 4: launch_unpack_variant<4, PARAM, 1>(a, g.slots, vec4, grid, s); break;
+      default: launch_unpack_variant<8, PARAM, 1>(a, g.slots, vec4, grid, s); break;
+    }
   }
   return launch_status();
 }

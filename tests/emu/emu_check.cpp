@@ -505,6 +505,19 @@ static void check_colsum(int64_t N, int64_t K, std::mt19937& rng) {
           "moments N=%lld K=%lld col %lld", (long long)N, (long long)K, (long long)k);
 }
 
+// Unpack alone on random packed bytes, at sizes that take the several-rows-per-lane-group form of the kernel.
+static void check_unpack_only(int64_t N, int64_t G, int bits, std::mt19937& rng) {
+  const int64_t nb = exact_packed_nbytes(N, G, bits);
+  Buf<uint8_t> packed(nb);
+  Buf<float> sc(N), mn(N), out(N * G), want(N * G);
+  for (int64_t i = 0; i < nb; ++i) packed[i] = static_cast<uint8_t>(rng());
+  std::uniform_real_distribution<float> ud(0.5f, 40.f);
+  for (int64_t i = 0; i < N; ++i) { sc[i] = ud(rng); mn[i] = ud(rng) - 20.f; }
+  oracle_unpack(packed.p, bits, sc.p, mn.p, N, G, want.p);
+  const int rc = exact_unpack_f32(packed.p, bits, sc.p, mn.p, N, G, out.p, nullptr);
+  CHECK(rc == 0 && std::memcmp(out.p, want.p, N * G * 4) == 0, "unpack alone differs N=%ld G=%ld bits=%d", (long)N, (long)G, bits);
+}
+
 static void check_dw(int64_t N, int64_t K, int64_t D, int64_t pad, std::mt19937& rng) {
   std::uniform_int_distribution<int> id(-3, 3);
   const int64_t ldy = K + pad, ldx = D + 2 * pad;
@@ -537,6 +550,16 @@ int main(int argc, char** argv) {
   if (mode == "rp") {  // the projection kernels only
     for (auto& s : kRpShapes) check_rp(s[0], s[1], s[2], rng);
     std::printf("rp shapes ok (failures so far %d)\n", g_fail);
+    return g_fail != 0;
+  }
+  if (mode == "unpack") {  // the several-rows form of the unpack kernel
+    for (int bits : {1, 2, 4, 8}) {
+      check_unpack_only(8229, 256, bits, rng);
+      check_unpack_only(65571, 32, bits, rng);
+      check_unpack_only(16397, 100, bits, rng);
+      check_unpack_only(131077, 8, bits, rng);
+    }
+    std::printf("unpack sizes ok (failures so far %d)\n", g_fail);
     return g_fail != 0;
   }
   if (mode == "dw") {  // the weight-gradient kernels only

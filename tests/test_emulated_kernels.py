@@ -45,6 +45,23 @@ def test_pack_unpack(bits, N, G):
     assert np.array_equal(e.pack(x, mn, want[4], bits, None, seed, off), got)
 
 
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("N,G", [(8229, 256), (65571, 32), (16397, 100), (8195, 1024), (131077, 8)])
+def test_unpack_with_several_rows_per_lane_group(bits, N, G):
+    """Activations large enough for the kernel form in which a lane group takes
+    four consecutive rows (all loads issued first): every value against the
+    oracle, with a ragged last group of rows, for fp32 and bf16 scale / min."""
+    rng = np.random.default_rng(N + G + bits)
+    packed = rng.integers(0, 256, o.packed_nbytes(N, G, bits), dtype=np.uint8)
+    scale = (rng.random(N) * 40 + 0.5).astype(F32)
+    mn = rng.standard_normal(N).astype(F32)
+    got = e.unpack(packed, bits, scale, mn, N, G)
+    assert np.array_equal(got.view(np.uint32), o.unpack_single_precision(packed, bits, scale, mn, N, G).view(np.uint32))
+    sbf, mbf = o.bf16_round(scale)[0], o.bf16_round(mn)[0]
+    got = e.unpack(packed, bits, sbf, mbf, N, G, bf16=True)
+    assert np.array_equal(got.view(np.uint32), o.dequantize_activation(packed, bits, sbf, mbf, (N, G)).view(np.uint32))
+
+
 def test_unpack_extreme_scales_take_the_division_path():
     # scales outside [2^-64, 2^64], inf and nan rows use the per-element IEEE division
     N, G, bits = 16, 24, 8
