@@ -294,13 +294,16 @@ def train_epochs(model, x, adj, labels, train_idx, epochs, warmup, lr=0.01):
 
 
 def epoch_algorithmic_bytes(kind, n, nnz, feat, hidden, classes, layers, bits, kept_frac, batch_norm, idx_bytes=4):
-    """Compulsory memory traffic of one training epoch's kernels on the
-    compression / aggregation path, as a list of (what, bytes): every operand
-    read once and every result written once per kernel, with the library's
-    default fusions (ReLU + dropout (+ batch norm) + quantise in one pass where
-    no projection is configured, projection + quantise in one pass otherwise).
-    Loss, optimiser and the small per-column vectors are left out.  This is
-    the numerator of the epoch's roofline fraction."""
+    """Compulsory memory traffic of one training epoch as a list of (what,
+    bytes): for every step of the algorithm as this library executes it by
+    default (one-node GCN / SAGE layers with the sparse product on the narrower
+    side, ReLU + dropout (+ batch norm) + quantise in one pass, projection +
+    quantise in one pass, second GEMMs accumulating into the first's result),
+    every operand read once and every result written once.  Passes that exist
+    only because two kernels were not fused -- adding a bias, adding two GEMM
+    results -- are NOT counted: they are not part of the algorithm.  Loss,
+    optimiser and the small per-column vectors are left out.  This is the
+    numerator of the epoch's roofline fraction."""
     f4 = 4 * n
     widths = [feat] + [hidden] * (layers - 1) + [classes]
     items = []
@@ -320,12 +323,13 @@ def epoch_algorithmic_bytes(kind, n, nnz, feat, hidden, classes, layers, bits, k
     for l in range(layers):
         cin, cout, last = widths[l], widths[l + 1], l == layers - 1
         needs_dx = l > 0
+        k = kept(cin)
         if kind == "gcn":
-            if l == 0 or kept_frac < 1.0:
-                add(f"L{l} quantise input", f4 * cin + packed(kept(cin)))
-            add(f"L{l} GEMM X W^T", f4 * cin + f4 * cout)
-            add(f"L{l} SpMM forward", spmm(cout, True))
-            add(f"L{l} bias add", 2 * f4 * cout)
+            if l == 0 or kept_frac < 1.0:                 # later layers get their copy from the fused pass before them
+                add(f"L{l} quantise input", f4 * cin + packed(k))
+            narrow = min(cin, cout)
+            add(f"L{l} SpMM forward (width {narrow})", spmm(narrow, True))
+            add(f"L{l} GEMM with W^T", f4 * cin + f4 * cout)
             if not last:
                 if batch_norm:
                     add(f"L{l} quantise batch-norm input", f4 * cout + packed(cout))
@@ -337,30 +341,39 @@ def epoch_algorithmic_bytes(kind, n, nnz, feat, hidden, classes, layers, bits, k
                     add(f"L{l} backward: norm column sums", 2 * f4 * cout)
                     add(f"L{l} backward: norm element-wise", 3 * f4 * cout)
             add(f"L{l} backward: bias gradient", f4 * cout)
-            add(f"L{l} backward: SpMM transpose", spmm(cout, True))
-            add(f"L{l} backward: restore input", packed(kept(cin)) + f4 * kept(cin))
-            add(f"L{l} backward: dW", f4 * cout + f4 * kept(cin))
-            if needs_dx:
-                add(f"L{l} backward: dX", f4 * cout + f4 * cin)
+            add(f"L{l} backward: restore input", packed(k) + f4 * k)
+            if needs_dx or k >= cout:
+                add(f"L{l} backward: SpMM transpose (width {cout})", spmm(cout, True))
+                add(f"L{l} backward: dW", f4 * cout + f4 * k)
+                if needs_dx:
+                    add(f"L{l} backward: dX", f4 * cout + f4 * cin)
+            else:                                         # first layer: the sparse product runs on the kept copy
+                add(f"L{l} backward: SpMM on the kept copy (width {k})", spmm(k, True))
+                add(f"L{l} backward: dW", f4 * cout + f4 * k)
         else:
-            add(f"L{l} project + quantise input (shared copy)", f4 * cin + packed(kept(cin)))
-            add(f"L{l} SpMM mean forward", spmm(cin, False))
-            add(f"L{l} project + quantise aggregate", f4 * cin + packed(kept(cin)))
-            add(f"L{l} GEMM lin_l", f4 * cin + f4 * cout)
-            add(f"L{l} GEMM lin_r", f4 * cin + f4 * cout)
-            add(f"L{l} add", 3 * f4 * cout)
+            add(f"L{l} project + quantise input (shared copy)", f4 * cin + packed(k))
+            if kept_frac < 1.0 and k + cout < cin:        # aggregate x [R | W_l^T]
+                width = k + cout
+                add(f"L{l} GEMM x [R | W_l^T]", f4 * cin + f4 * width)
+                add(f"L{l} SpMM mean forward (width {width})", spmm(width, False))
+                add(f"L{l} quantise aggregate copy", f4 * k + packed(k))
+                add(f"L{l} GEMM lin_r (accumulating)", f4 * cin + f4 * cout)
+            else:
+                add(f"L{l} SpMM mean forward (width {cin})", spmm(cin, False))
+                add(f"L{l} project + quantise aggregate", f4 * cin + packed(k))
+                add(f"L{l} GEMM lin_l", f4 * cin + f4 * cout)
+                add(f"L{l} GEMM lin_r (accumulating)", f4 * cin + f4 * cout)
             if not last:
                 add(f"L{l} ReLU + dropout", 2 * f4 * cout + n * cout / 8)
                 add(f"L{l} backward: mask", 2 * f4 * cout + n * cout / 8)
             add(f"L{l} backward: bias gradient", f4 * cout)
             for which in ("lin_l", "lin_r"):
-                add(f"L{l} backward: restore {which} input", packed(kept(cin)) + f4 * kept(cin))
-                add(f"L{l} backward: dW {which}", f4 * cout + f4 * kept(cin))
-                if needs_dx:
-                    add(f"L{l} backward: dX {which}", f4 * cout + f4 * cin)
+                add(f"L{l} backward: restore {which} input", packed(k) + f4 * k)
+                add(f"L{l} backward: dW {which}", f4 * cout + f4 * k)
             if needs_dx:
-                add(f"L{l} backward: SpMM transpose", spmm(cin, True))
-                add(f"L{l} backward: gradient sum", 3 * f4 * cin)
+                narrow = min(cin, cout)
+                add(f"L{l} backward: SpMM transpose (width {narrow})", spmm(narrow, True))
+                add(f"L{l} backward: dX (two GEMMs, the second accumulating)", 2 * f4 * cout + f4 * cin)
     return items
 
 
