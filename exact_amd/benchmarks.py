@@ -524,7 +524,7 @@ def _profile_target(argv=None):
     `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
 
         python -m exact_amd.benchmarks pack --bits 2 --reps 100
-        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy,probe} ...
+        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy,probe,dw} ...
         python -m exact_amd.benchmarks epoch --config cfg3_gcn_int2 --epochs 5
 
     `copy` is a plain device-to-device copy of the same [rows, cols] fp32 tensor
@@ -542,7 +542,10 @@ def _profile_target(argv=None):
         return _epoch_main(argv[1:])
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
     ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "relu_dropout_pack", "bn_relu_dropout_pack", "rp_fwd", "rp_bwd",
-                                      "rp_pack", "spmm", "copy", "probe"])
+                                      "rp_pack", "spmm", "copy", "probe", "dw"])
+    ap.add_argument("--fp32-cores", action="store_true", help="dw only: the fp32 matrix-core kernel instead of the bf16 one")
+    ap.add_argument("--cold", action="store_true",
+                    help="unpack only: every launch reads another copy of the packed stream (24 copies, none of it cached)")
     ap.add_argument("--rp-path", choices=["fp32", "split", "signs"], default="signs",
                     help="rp_* only: the fp32 matrix-core instruction on a Gaussian matrix, the bf16 instruction on split "
                          "operands (Gaussian matrix), or on the signs of a +-1/sqrt(k) matrix (the default path)")
@@ -589,11 +592,15 @@ def _profile_target(argv=None):
         rowptr, col, value = adj.csr()
         spmm_x = torch.randn((n_nodes, args.width or G), generator=gen, device=dev)
         spmm_reduce = "sum" if kind == "gcn" else "mean"
+    packs = [packed] + [packed.clone() for _ in range(23)] if args.cold else [packed]
+    dw_out = torch.empty((G, G), device=dev)
+    dw_entry = L.exact_linear_dw_f32 if args.fp32_cores else L.exact_linear_dw_bf16_f32
     fns = {
+        "dw": lambda i: dw_entry(xs[i % 3].data_ptr(), G, xs[(i + 1) % 3].data_ptr(), G, N, G, G, dw_out.data_ptr(), sp),
         "pack": lambda i: L.exact_minmax_pack_f32(xs[i % 3].data_ptr(), noise.data_ptr() if noise is not None else None, 1,
                                                   i, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),
                                                   mbf.data_ptr(), sp),
-        "unpack": lambda i: L.exact_unpack_bf16param_f32(packed.data_ptr(), b, sbf.data_ptr(), mbf.data_ptr(), N, G,
+        "unpack": lambda i: L.exact_unpack_bf16param_f32(packs[i % len(packs)].data_ptr(), b, sbf.data_ptr(), mbf.data_ptr(), N, G,
                                                          outs[i % 3].data_ptr(), sp),
         "relu": lambda i: L.exact_relu_fwd_f32(xs[i % 3].data_ptr(), N * G, outs[i % 3].data_ptr(), mask.data_ptr(), sp),
         "dropout": lambda i: L.exact_dropout_fwd_f32(xs[i % 3].data_ptr(), None, 1, i, 0.5, N * G, outs[i % 3].data_ptr(),

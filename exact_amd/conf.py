@@ -89,6 +89,12 @@ _EXTRA_FIELDS = {
     # also switched on by torch.use_deterministic_algorithms(True).  The default
     # kernel balances hub rows across wavefronts and adds their parts atomically.
     "deterministic_spmm": False,
+    # Column sums, weight gradients, batch statistics and the batch-norm
+    # backward reductions combine partial results with fp32 atomics (no fixed
+    # summation order: the last bits vary from run to run).  True sends all four
+    # to the framework's own, reproducible routines, as
+    # torch.use_deterministic_algorithms(True) does.
+    "deterministic_reductions": False,
 }
 
 

@@ -9,15 +9,23 @@ from ..conf import config
 from . import _checks
 
 
+def _atomics_allowed():
+    """The library's reductions meet in memory through atomics; both the
+    framework's deterministic mode and config.deterministic_reductions ask for
+    reproducible sums instead."""
+    return not (torch.are_deterministic_algorithms_enabled() or config.deterministic_reductions)
+
+
 def column_sums(matrix):
     """`matrix.sum(0)` of a 2-D tensor.  fp32 device matrices go through the
     library's streaming kernel (the framework's reduction runs far off the
     memory roofline for narrow matrices: 19 ms for [2.4M, 47]); its atomics
-    fix no summation order, so deterministic mode and everything else keep the
-    framework's reduction."""
+    fix no summation order, so deterministic mode
+    (config.deterministic_reductions or the framework's own switch) and
+    everything else keep the framework's reduction."""
     usable = (matrix.dim() == 2 and matrix.dtype == torch.float32 and _checks.on_device(matrix)
               and matrix.is_contiguous() and 0 < matrix.shape[1] <= 256 and matrix.shape[0] >= 4096
-              and not torch.are_deterministic_algorithms_enabled())
+              and _atomics_allowed())
     if not usable:
         return matrix.sum(0)
     out = torch.empty(matrix.shape[1], dtype=torch.float32, device=matrix.device)
@@ -31,16 +39,17 @@ def batch_statistics(matrix):
     """(biased variance, mean) of every column of a 2-D tensor, what
     torch.var_mean(matrix, dim=0, unbiased=False) returns.  Tall fp32 device
     matrices of at most 256 columns take the library's one-pass kernel (moments
-    centred on the mean of the first 256 rows, close enough to the column mean
-    that the difference of the two moments loses no digits); everything else
-    the framework's reduction."""
-    usable = (matrix.dim() == 2 and matrix.dtype == torch.float32 and matrix.is_cuda and matrix.is_contiguous()
+    centred on the mean of 256 rows spread evenly over the matrix -- also for
+    sorted or clustered rows a centre within a fraction of a standard deviation
+    of the column mean, so that the difference of the two moments loses no
+    digits); everything else the framework's reduction."""
+    usable = (matrix.dim() == 2 and matrix.dtype == torch.float32 and _checks.on_device(matrix) and matrix.is_contiguous()
               and 0 < matrix.shape[1] <= 256 and matrix.shape[0] >= 4096
-              and not torch.are_deterministic_algorithms_enabled())
+              and _atomics_allowed())
     if not usable:
         return torch.var_mean(matrix, dim=0, unbiased=False)
     N, K = matrix.shape
-    center = matrix[:256].mean(0)
+    center = matrix[::N // 256][:256].mean(0)
     sums = torch.empty((2, K), dtype=torch.float32, device=matrix.device)
     rc = _lib.lib().exact_col_moments_f32(_checks.ptr(matrix), _checks.ptr(center), N, K, _checks.ptr(sums[0]),
                                           _checks.ptr(sums[1]), _checks.stream_ptr(matrix))
@@ -61,7 +70,7 @@ def weight_gradient(grad_output, input):  # noqa: A002
               and 0 < grad_output.shape[1] <= 1024 and 0 < input.shape[1] <= 1024
               and grad_output.stride(1) == 1 and input.stride(1) == 1
               and grad_output.stride(0) >= grad_output.shape[1] and input.stride(0) >= input.shape[1]
-              and not torch.are_deterministic_algorithms_enabled())
+              and _atomics_allowed())
     if not usable:
         return grad_output.t().mm(input)
     N, K = grad_output.shape
@@ -99,11 +108,17 @@ def native_batch_norm_backward(grad_out, input, weight, running_mean, running_va
     the framework's batch_norm_backward_elemt, which computes
       dx = (dy - sum_dy / N - (x - mean) * invstd^2 * sum_dy_xmu / N) * invstd * weight
     exactly as the one-call routine does."""
+    def stat_ok(t, optional=False):
+        if t is None:
+            return optional
+        return t.dtype == torch.float32 and t.device == grad_out.device and t.numel() == grad_out.shape[1]
+
     fast = (train and grad_out.dim() == 2 and grad_out.is_cuda and grad_out.dtype == torch.float32
-            and input.dtype == torch.float32 and grad_out.is_contiguous() and input.is_contiguous()
-            and grad_out.shape[0] >= 4096 and 0 < grad_out.shape[1] <= 256 and grad_out.shape == input.shape
-            and save_mean is not None and save_invstd is not None and save_mean.dtype == torch.float32
-            and not torch.are_deterministic_algorithms_enabled())
+            and input.dtype == torch.float32 and input.device == grad_out.device
+            and grad_out.is_contiguous() and input.is_contiguous()
+            and 4096 <= grad_out.shape[0] < 2 ** 31 and 0 < grad_out.shape[1] <= 256 and grad_out.shape == input.shape
+            and stat_ok(save_mean) and stat_ok(save_invstd) and stat_ok(weight, optional=True)
+            and _atomics_allowed())
     if not fast:
         return torch.ops.aten.native_batch_norm_backward(grad_out, input, weight, running_mean, running_var,
                                                          save_mean, save_invstd, train, eps, list(output_mask))

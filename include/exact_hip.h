@@ -209,8 +209,9 @@ int exact_bn_backward_reduce_f32(const float *dy, const float *x, const float *m
 int exact_col_moments_f32(const float *x, const float *center, int64_t N, int64_t K, float *sum_d, float *sum_d2,
                           void *stream);
 
-/* Measurement aid with no counterpart in the reference: the memory traffic of the
- * pack kernel without its arithmetic.  Every lane reads 64 bytes of x (n floats,
+/* FOR BENCHMARKS ONLY -- not part of the operator interface; no product code calls it and a binding of the
+ * reference's operators has no use for it.  Measurement aid with no counterpart in the reference: the memory
+ * traffic of the pack kernel without its arithmetic.  Every lane reads 64 bytes of x (n floats,
  * whole tiles of 4096 floats; the remainder is not touched) and writes
  * out_bytes (0, 2, 4, 8 or 16: what 1 / 2 / 4 / 8 bits per element make of 16
  * elements) to `out`, which holds (n / 16) * out_bytes bytes (at least 16).  x

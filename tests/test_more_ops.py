@@ -644,6 +644,56 @@ def test_batch_statistics_match_var_mean(cuda, N, K):
     assert ((var.double() - want_var) / want_var).abs().max().item() < 1e-5
 
 
+def test_batch_statistics_of_sorted_rows(backend):
+    """Rows sorted by value, the first 256 of them many standard deviations from
+    the column mean: the moments stay centred near the mean (a sample spread over
+    all rows), so the variance keeps its digits."""
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(6000, 9, generator=g) * 0.01 + torch.linspace(-50.0, 50.0, 6000)[:, None]).sort(0).values.contiguous()
+    var, mean = bf.batch_statistics(x.to(backend))
+    want_var, want_mean = torch.var_mean(x.double(), dim=0, unbiased=False)
+    assert (mean.cpu().double() - want_mean).abs().max().item() < 1e-4
+    assert ((var.cpu().double() - want_var) / want_var).abs().max().item() < 1e-5
+
+
+def test_reductions_keep_the_framework_routines_on_request(backend, monkeypatch):
+    """config.deterministic_reductions = True: no atomics-combined kernel is
+    called for column sums, weight gradients and batch statistics."""
+    from exact_amd import _lib
+    from exact_amd.conf import config
+    from exact_amd.cpp_extension import backward_func as bf
+    g = torch.Generator().manual_seed(12)
+    dy, x = torch.randn(16500, 8, generator=g).to(backend), torch.randn(16500, 12, generator=g).to(backend)
+    free = (bf.column_sums(dy), bf.weight_gradient(dy, x), bf.batch_statistics(x))
+    monkeypatch.setattr(config, "deterministic_reductions", True)
+
+    def no_library():
+        raise AssertionError("a library kernel was asked for")
+    monkeypatch.setattr(_lib, "lib", no_library)
+    fixed = (bf.column_sums(dy), bf.weight_gradient(dy, x), bf.batch_statistics(x))
+    assert torch.equal(fixed[0], dy.sum(0)) and torch.equal(fixed[1], dy.t().mm(x))
+    assert torch.allclose(free[0], fixed[0], atol=1e-3) and torch.allclose(free[1], fixed[1], atol=1e-3)
+    assert torch.allclose(free[2][0], fixed[2][0], atol=1e-5) and torch.allclose(free[2][1], fixed[2][1], atol=1e-5)
+
+
+def test_batch_norm_backward_refuses_mismatched_statistics_for_the_fast_path(backend, monkeypatch):
+    """Statistics of the wrong length, type or device never reach the kernel:
+    the call falls through to the framework's routine (which raises or handles
+    them by its own rules)."""
+    from exact_amd import _lib
+    from exact_amd.cpp_extension import backward_func as bf
+    seen = []
+    monkeypatch.setattr(torch.ops.aten, "native_batch_norm_backward", lambda *a: seen.append(a) or "framework")
+    monkeypatch.setattr(_lib, "lib", lambda: (_ for _ in ()).throw(AssertionError("kernel reached")))
+    dy, x = torch.zeros(5000, 8).to(backend), torch.zeros(5000, 8).to(backend)
+    ok = torch.ones(8).to(backend)
+    for mean, invstd, weight in ((ok[:7], ok, ok), (ok, ok.double(), ok), (ok, ok, torch.ones(9).to(backend)), (None, ok, ok),
+                                 (ok, ok.cpu() if ok.is_cuda else ok[:3], ok)):
+        assert bf.native_batch_norm_backward(dy, x, weight, None, None, mean, invstd, True, 1e-5, (True, True, True)) == "framework"
+    assert len(seen) == 5
+
+
 def test_sparse_product_with_row_strides(backend):
     """The dense operand as a column slice of a wider buffer (unit column
     stride, longer row stride) and the padded copy the shim makes of wide,

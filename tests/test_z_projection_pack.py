@@ -1,7 +1,11 @@
 """input2rp + quantize_activation as one launch (exact_rp_minmax_pack_f32) on
 the Python side, both back ends: identical to the two calls it replaces
-(reference ops.py:141-149, layers.py:153-159).  The kernel is pinned bit for
-bit against the oracle in test_emulated_kernels.py."""
+(reference ops.py:141-149, layers.py:153-159).  Both sides of the comparison
+here are this library's own kernels: it shows that the host side's fused and
+unfused routes agree, not that either is right.  The kernel itself is pinned
+bit for bit against the oracle in test_emulated_kernels.py (emulator) and
+test_gpu_rp.py (GPU, through the C ABI, every matrix-core path).  Collected
+late on purpose: it switches config.fuse_epilogue and the projection sources."""
 import pytest
 import torch
 import torch.nn.functional as F
