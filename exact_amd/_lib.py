@@ -73,6 +73,9 @@ SIGNATURES = {
     "exact_rp_bwd_bf16_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_ptr]),
     "exact_rp_minmax_pack_bf16_f32": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_u64, _c_u64, _c_i64, _c_i64, _c_i64,
                                                _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
+    "exact_tall_gemm_table_nbytes": (_c_i64, [_c_i64, _c_i64]),
+    "exact_tall_gemm_prepare_bf16": (_c_int, [_c_ptr, _c_i64, _c_int, _c_i64, _c_i64, _c_ptr, _c_ptr]),
+    "exact_tall_gemm_bf16_f32": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr]),
 }
 
 _lib = None

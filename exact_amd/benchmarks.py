@@ -17,6 +17,7 @@ import torch.nn.functional as F
 from . import ops
 from .conf import QuantizationConfig, config
 from .cpp_extension import quantization as extq
+from .cpp_extension import backward_func as ext_backward_func
 from .cpp_extension import spmm as ext_spmm
 from .models import GCN, SAGE
 from .module import QModule
@@ -220,6 +221,29 @@ def kernel_extras(x, log):
         q, R, _ = ops.project_and_quantize(x, None)
         t = event_time(lambda: ops.rp2input(ops.dequantize_activation(q, xr_small.shape), x.shape, R))
         out["rp_decompress_int2"] = {"us": t * 1e6}
+        # the dense products of a layer: x W^T + b and dY^T x at 256 x 256, library kernels against the framework's GEMM
+        w = torch.randn(G, G, device=x.device) / G ** 0.5
+        bias = torch.randn(G, device=x.device)
+        flops = 2.0 * N * G * G
+        gemm_bytes = 8 * N * G + 4 * G * G
+        config.tall_gemm_max_cols = 4096
+        w40 = torch.randn(40, G, device=x.device) / G ** 0.5
+        for cores in ("bf16", "fp32"):
+            config.matrix_cores = cores
+            t = event_time(lambda: ext_backward_func.tall_matmul(nx(), w40, transposed=True))
+            out[f"linear_forward_{G}x40_{cores}"] = {"us": t * 1e6, "TFLOP/s": 2.0 * N * G * 40 / t / 1e12,
+                                                     "what": "six bf16 matrix-core products per fp32 product (library kernel)"
+                                                     if cores == "bf16" else "the framework's fp32 GEMM"}
+            t = event_time(lambda: ext_backward_func.tall_matmul(nx(), w, transposed=True, bias=bias))
+            out[f"linear_forward_{G}x{G}_{cores}"] = {"us": t * 1e6, "TFLOP/s": flops / t / 1e12, "GB/s": gemm_bytes / t / 1e9,
+                                                      "algo_bytes": gemm_bytes,
+                                                      "what": "six bf16 matrix-core products per fp32 product (library kernel)"
+                                                      if cores == "bf16" else "the framework's fp32 GEMM (addmm)"}
+            t = event_time(lambda: ext_backward_func.weight_gradient(nx(), nx()))
+            out[f"weight_gradient_{G}x{G}_{cores}"] = {"us": t * 1e6, "TFLOP/s": flops / t / 1e12,
+                                                       "what": "library kernel, bf16 instruction on split operands" if cores == "bf16"
+                                                       else "library kernel, fp32 instruction"}
+        config.matrix_cores = "bf16"
         for name, v in out.items():
             if "GB/s" in v:
                 v["frac_hbm_peak"] = v["GB/s"] / HBM_PEAK_GBS

@@ -95,6 +95,13 @@ _EXTRA_FIELDS = {
     # to the framework's own, reproducible routines, as
     # torch.use_deterministic_algorithms(True) does.
     "deterministic_reductions": False,
+    # The dense products of a layer (x W^T, dY W) go to the library's bf16
+    # matrix-core kernel (config.matrix_cores == "bf16") from this many rows on;
+    # shorter operands keep the framework's GEMM, which is as fast there.
+    "tall_gemm_min_rows": 16384,
+    # ... and up to this many output columns: measured against the framework's
+    # fp32 GEMM the kernel is 20 - 25 % faster at 40 - 47 columns and equal at 256.
+    "tall_gemm_max_cols": 64,
 }
 
 

@@ -85,10 +85,78 @@ def weight_gradient(grad_output, input):  # noqa: A002
     return out
 
 
+# ---- the dense products of a layer on the bf16 matrix cores ---------------------
+def _gemm_table(matrix, transposed, D, K):
+    """Operand fragments of `matrix` for exact_tall_gemm_bf16_f32, remembered on the
+    tensor until it changes (a weight is prepared once per optimiser step)."""
+    key = (bool(transposed), matrix._version, matrix.data_ptr(), tuple(matrix.shape), matrix.stride(0))
+    cached = getattr(matrix, "_exact_gemm_table", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    L = _lib.lib()
+    table = torch.empty(int(L.exact_tall_gemm_table_nbytes(D, K)), dtype=torch.uint8, device=matrix.device)
+    rc = L.exact_tall_gemm_prepare_bf16(_checks.ptr(matrix), matrix.stride(0), int(bool(transposed)), D, K, _checks.ptr(table),
+                                        _checks.stream_ptr(matrix))
+    _lib.check(rc, "tall_matmul (prepare)")
+    try:
+        matrix._exact_gemm_table = (key, table)
+    except AttributeError:
+        pass
+    return table
+
+
+def tall_matmul(x, matrix, transposed=False, bias=None, addend=None, into=None):
+    """x[N, D] . M (+ bias[K]) (+ addend[N, K]) -> [N, K], where M = `matrix`
+    ([D, K]) or, with transposed=True, the transpose of `matrix` ([K, D]: a weight
+    as F.linear holds it).  `into` names the result tensor; it may be `addend`
+    itself (accumulate in place).  Tall fp32 device operands with a narrow result
+    (config.tall_gemm_min_rows, config.tall_gemm_max_cols) take the library's
+    kernel (six bf16 matrix-core products per fp32 product, fp32 accuracy,
+    reproducible; config.matrix_cores == "bf16"); everything else the
+    framework's GEMM."""
+    M = matrix.t() if transposed else matrix
+    usable = (config.matrix_cores == "bf16" and x.dim() == 2 and matrix.dim() == 2 and x.dtype == torch.float32
+              and matrix.dtype == torch.float32 and _checks.on_device(x) and _checks.on_device(matrix)
+              and x.shape[1] == M.shape[0] and x.shape[0] >= config.tall_gemm_min_rows and x.shape[1] % 4 == 0
+              and 0 < x.shape[1] <= 4096 and 0 < M.shape[1] <= min(4096, config.tall_gemm_max_cols) and x.is_contiguous() and x.data_ptr() % 16 == 0
+              and matrix.stride(1) == 1 and matrix.stride(0) >= matrix.shape[1]
+              and (bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == M.shape[1]
+                                    and _checks.on_device(bias)))
+              and (addend is None or (addend.dtype == torch.float32 and addend.dim() == 2 and addend.stride(1) == 1
+                                      and addend.shape == (x.shape[0], M.shape[1]) and _checks.on_device(addend)))
+              and (into is None or (into.dtype == torch.float32 and into.dim() == 2 and into.stride(1) == 1
+                                    and into.shape == (x.shape[0], M.shape[1]) and _checks.on_device(into)))
+              and not (torch.is_grad_enabled() and (x.requires_grad or matrix.requires_grad
+                                                    or (bias is not None and bias.requires_grad)
+                                                    or (addend is not None and addend.requires_grad))))
+    if not usable:
+        if addend is not None:
+            out = torch.addmm(addend, x, M) if into is None or into is not addend else addend.addmm_(x, M)
+            if bias is not None:
+                out += bias
+        else:
+            out = x.mm(M) if bias is None else torch.addmm(bias, x, M)
+        if into is not None and into is not out:
+            into.copy_(out)
+            out = into
+        return out
+    N, D = x.shape
+    K = M.shape[1]
+    out = into if into is not None else torch.empty((N, K), dtype=torch.float32, device=x.device)
+    table = _gemm_table(matrix, transposed, D, K)
+    rc = _lib.lib().exact_tall_gemm_bf16_f32(_checks.ptr(x), _checks.ptr(table), N, D, K,
+                                             _checks.ptr(bias) if bias is not None else None,
+                                             _checks.ptr(addend) if addend is not None else None,
+                                             addend.stride(0) if addend is not None else K, _checks.ptr(out), out.stride(0),
+                                             _checks.stream_ptr(x))
+    _lib.check(rc, "tall_matmul")
+    return out
+
+
 def linear_backward(grad_output, input, weight, bias, need_input_grad=True):  # noqa: A002
     """backward_func.cc:83-93.  `need_input_grad=False` leaves out the product
     the caller would discard (the reference forms all three regardless)."""
-    grad_input = grad_output.mm(weight) if need_input_grad else None
+    grad_input = tall_matmul(grad_output, weight) if need_input_grad else None
     grad_weight = weight_gradient(grad_output, input)
     grad_bias = column_sums(grad_output) if bias is not None else None
     return grad_input, grad_weight, grad_bias

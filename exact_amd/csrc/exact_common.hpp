@@ -78,6 +78,37 @@ __device__ __forceinline__ void philox_uniform8(const Philox4& r, float (&u)[8])
   u[7] = u16_to_uniform(r.w >> 16);
 }
 
+// ---- round and clamp of the quantiser -------------------------------------------
+// quantization_cuda_kernel.cu:89-90 turns t = (x - min) * scale + noise into
+// uint8(__float2int_rn(fmaxf(t - 0.5f, 0.f))).  When scale and min are the row's
+// own, t is below 2^bits + 2, or +inf (a row whose spread is so small that its
+// reciprocal overflows), or NaN (0 * inf in a constant row).  For those the same
+// byte is the low byte of the bit pattern of  med3(t, 0.5, 511.5) + (2^23 - 0.5):
+// t - 0.5 is exact in fp32 whenever t >= 0.5 (a multiple of ulp(t) of smaller
+// magnitude), so the sum has the exact value 2^23 + (t - 0.5) in [2^23, 2^24),
+// where fp32 holds the integers only -- the one rounding of the addition is the
+// round-to-nearest-even onto the integers that __float2int_rn performs, and the
+// low mantissa bits are that integer.  t < 0.5 gives 2^23 exactly, code 0, as
+// fmaxf(.., 0) does, and so does NaN (v_med3_f32 with a NaN operand returns the
+// minimum of the others); +inf is clamped to 511, low byte 0xFF, the low byte of
+// the INT_MAX that the saturating conversion returns.  Two instructions instead
+// of five.  Callers whose t is not bounded (scale and min supplied from outside)
+// keep the written-out form, which saturates at every magnitude.
+__device__ __forceinline__ uint32_t code_in_low_byte(float t) {
+  return __float_as_uint(__builtin_amdgcn_fmed3f(t, 0.5f, 511.5f) + 8388607.5f);
+}
+// __float2int_rn of a value that is not negative and not a NaN, every magnitude:
+// cvt.rni.s32.f32 clamps to the int32 range (a plain cast of +inf is undefined)
+__device__ __forceinline__ uint32_t float2int_rn_sat(float t) {
+  return t >= 2147483648.f ? 0x7FFFFFFFu : static_cast<uint32_t>(static_cast<int>(rintf(t)));
+}
+// the low bytes of four words as one word, a in byte 0 (three v_perm_b32)
+__device__ __forceinline__ uint32_t low_bytes4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const uint32_t ab = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);
+  const uint32_t cd = __builtin_amdgcn_perm(d, c, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
 // ---- bf16 ------------------------------------------------------------------
 // fp32 -> bf16 bits, round to nearest even (what Tensor.to(torch.bfloat16)
 // does at ops.py:80-81 of the reference).

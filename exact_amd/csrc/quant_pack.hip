@@ -20,9 +20,15 @@
 // operations and this file is compiled with -ffp-contract=off, so the result
 // is the unfused expression of the reference source.
 
+#include <cmath>
+
 #include "exact_common.hpp"
 
 namespace exact {
+
+// offsets inside the rows of one workgroup: 32 bits where the rows are known to be short
+template <bool NARROW> struct OffsetType { using type = int64_t; };
+template <> struct OffsetType<true> { using type = uint32_t; };
 
 // ---------------------------------------------------------------------------
 // loads / stores of one oct with `nv` (0..8) valid leading elements
@@ -94,21 +100,27 @@ __device__ __forceinline__ int swizzled_oct(int lir, int lpr, int k) {
   return (2 * k + (lir & 1)) * (lpr >> 1) + (lir >> 1);
 }
 
-template <int OPT>
-__device__ __forceinline__ void load_octs_swizzled(const float* __restrict__ seg, int lpr, int lir, float (&v)[OPT][8]) {
+template <int OPT, typename OFF>
+__device__ __forceinline__ void load_octs_swizzled(const float* __restrict__ base, OFF seg, int lpr, int lir,
+                                                   float (&v)[OPT][8]) {
+  // `base` is the same for the whole workgroup and `seg` (the lane's row segment, in floats from base) is
+  // 32 bits wide in the one-launch forms: the addresses then need no 64-bit vector arithmetic
   f32x4 q[2 * OPT];
 #pragma unroll
-  for (int i = 0; i < 2 * OPT; ++i) q[i] = nt_load4(seg + 4 * (i * lpr + lir));
+  for (int i = 0; i < 2 * OPT; ++i) q[i] = nt_load4(base + (seg + static_cast<OFF>(4 * (i * lpr + lir))));
   const bool odd = lir & 1;
 #pragma unroll
   for (int k = 0; k < OPT; ++k) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const float even_i = q[2 * k][c], odd_i = q[2 * k + 1][c];  // this lane's half of oct 2k' and of oct 2k' + 1
-      const float send = odd ? even_i : odd_i;
-      const float recv = __int_as_float(dpp_lanes<0xB1>(__float_as_int(send)));  // the neighbour's: lanes 2m <-> 2m + 1
-      v[k][c] = odd ? recv : even_i;       // first half: columns 0..3 of the oct (held by the even lane)
-      v[k][4 + c] = odd ? odd_i : recv;    // second half (held by the odd lane)
+      // this lane's half of oct 2k' (even_i) and of oct 2k' + 1 (odd_i); the even lane keeps oct 2k' and
+      // wants the neighbour's even_i, the odd lane keeps oct 2k' + 1 and wants the neighbour's odd_i
+      // (lanes 2m <-> 2m + 1; each select takes the neighbour's value through DPP in the same instruction)
+      const float even_i = q[2 * k][c], odd_i = q[2 * k + 1][c];
+      const float from_even = __int_as_float(dpp_lanes<0xB1>(__float_as_int(odd_i)));
+      const float from_odd = __int_as_float(dpp_lanes<0xB1>(__float_as_int(even_i)));
+      v[k][c] = odd ? from_even : even_i;       // first half: columns 0..3 of the oct (held by the even lane)
+      v[k][4 + c] = odd ? odd_i : from_odd;     // second half (held by the odd lane)
     }
   }
 }
@@ -136,6 +148,7 @@ struct PackArgs {
   // ACT form only: ReLU + dropout applied to x before the statistics
   const float* act_noise;  // nullable
   uint32_t act_seed_lo, act_seed_hi, act_off_lo, act_off_hi;
+  uint32_t act_keep_from;  // generator noise: an element is kept when its 16 random bits are >= this
   float p, pinv;
   float* y;                // activation output [N, G]
   uint8_t* mask_bytes;     // 1-bit mask of (x > 0) && keep, byte i / 8 holds elements i .. i + 7
@@ -172,15 +185,28 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   const int lane_in_row = t & (lpr - 1);
   const int row_local = t >> a.lpr_log2;
   const int rows_per_wg = kBlock >> a.lpr_log2;
-  const int64_t n = static_cast<int64_t>(blockIdx.x) * rows_per_wg + row_local;
-  const bool row_ok = n < a.N;
+  // Addresses are "first row of this workgroup" (the same for every lane: scalar registers) plus an offset
+  // inside the workgroup's rows, which fits 32 bits in the one-launch forms (G <= 1024) -- no 64-bit vector
+  // arithmetic there.  The two-step form (any G) keeps 64-bit offsets.
+  using off_t = typename OffsetType<FUSED>::type;
+  const int64_t row_base = static_cast<int64_t>(blockIdx.x) * rows_per_wg;
+  const int64_t rows_left = a.N - row_base;  // >= 1
+  const int rows_here = rows_left < rows_per_wg ? static_cast<int>(rows_left) : rows_per_wg;
+  const bool row_ok = row_local < rows_here;
+  const uint32_t n_lo = static_cast<uint32_t>(row_base) + static_cast<uint32_t>(row_local);  // N < 2^32
+  const off_t G = static_cast<off_t>(a.G);
+  const off_t row_off = static_cast<off_t>(row_local) * G;
+  const float* __restrict__ xw = HALF ? nullptr : a.x + row_base * a.G;
+  const half_t* __restrict__ hw = HALF ? reinterpret_cast<const half_t*>(a.x) + row_base * a.G : nullptr;
   const int oct_base = blockIdx.y * (lpr * OPT);  // 0 in the fused form
-  const int64_t row_off = n * a.G;
   // which octs of the row segment a lane owns: lane + k * lpr, or the row-contiguous assignment
-  const bool swz = FULL && VEC == 4 && !HALF && lpr >= 2;
+  // (whole rows of 16-byte aligned fp32 octs; the host launches those forms with lpr >= 2 only)
+  constexpr bool swz = FULL && VEC == 4 && !HALF;
   auto oct_of = [&](int lir, int k) {
     return oct_base + (swz ? swizzled_oct<OPT>(lir, lpr, k) : lir + k * lpr);
   };
+  // rows past the end re-read the last row and drop it
+  const off_t row_ld_off = static_cast<off_t>(row_ok ? row_local : rows_here - 1) * G + static_cast<off_t>(8 * oct_base);
 
   float v[OPT][8];
   int nv[OPT];
@@ -189,38 +215,42 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
     const int j = oct_of(lane_in_row, k);
     const int d0 = 8 * j;
     nv[k] = (row_ok && j < a.opr) ? min(8, a.G - d0) : 0;
-    if (swz) {
-      // all OPT octs at once, by every lane (the lanes of a pair trade halves): rows past the
-      // end re-read the last row and drop it
-      if constexpr (!HALF) {
-        if (k == 0) {
-          const int64_t n_ld = row_ok ? n : a.N - 1;
-          load_octs_swizzled<OPT>(a.x + n_ld * a.G + 8 * oct_base, lpr, lane_in_row, v);
-          if (!row_ok) {
+    if constexpr (swz) {
+      // all OPT octs at once, by every lane (the lanes of a pair trade halves)
+      if (k == 0) {
+        load_octs_swizzled<OPT, off_t>(xw, row_ld_off, lpr, lane_in_row, v);
+        if (!row_ok) {
 #pragma unroll
-            for (int kk = 0; kk < OPT; ++kk)
+          for (int kk = 0; kk < OPT; ++kk)
 #pragma unroll
-              for (int i = 0; i < 8; ++i) v[kk][i] = 0.f;
-          }
+            for (int i = 0; i < 8; ++i) v[kk][i] = 0.f;
         }
       }
     } else if (FULL && !row_ok) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[k][i] = 0.f;
     } else {
-      if constexpr (HALF) load_oct_half<VEC, FULL>(reinterpret_cast<const half_t*>(a.x) + row_off + d0, nv[k], v[k]);
-      else load_oct<VEC, FULL>(a.x + row_off + d0, nv[k], v[k]);
+      if constexpr (HALF) load_oct_half<VEC, FULL>(hw + (row_off + static_cast<off_t>(d0)), nv[k], v[k]);
+      else load_oct<VEC, FULL>(xw + (row_off + static_cast<off_t>(d0)), nv[k], v[k]);
     }
     if constexpr (ACT) {
       if (nv[k] > 0) {  // G % 8 == 0: a whole oct or nothing
-        const int64_t blk = (row_off + d0) >> 3;
+        // Philox block and mask byte of this oct: flat element index / 8 (G % 8 == 0)
+        const uint32_t g8 = static_cast<uint32_t>(a.G) >> 3;
+        const uint32_t blk_local = static_cast<uint32_t>(row_local) * g8 + static_cast<uint32_t>(j);
+        const int64_t blk = row_base * g8 + blk_local;
+        // keep[i]: the element's uniform exceeds p.  Supplied noise is compared as it is; the generator's
+        // uniform is (h + 0.5) / 65536 for 16 random bits h, exactly, so u > p  <=>  h >= act_keep_from
+        // (the host works the threshold out in double): no conversion per element
         float ud[8];
+        uint32_t hd[8];
         if constexpr (NOISE_IN) {
-          load_oct<VEC, true>(a.act_noise + row_off + d0, 8, ud);
+          load_oct<VEC, true>(a.act_noise + row_base * a.G + (row_off + static_cast<off_t>(d0)), 8, ud);
         } else {
           const Philox4 r = philox4x32_10(static_cast<uint32_t>(blk), static_cast<uint32_t>(blk >> 32),
                                           a.act_off_lo, a.act_off_hi, a.act_seed_lo, a.act_seed_hi);
-          philox_uniform8(r, ud);
+          hd[0] = r.x & 0xFFFFu; hd[1] = r.x >> 16; hd[2] = r.y & 0xFFFFu; hd[3] = r.y >> 16;
+          hd[4] = r.z & 0xFFFFu; hd[5] = r.z >> 16; hd[6] = r.w & 0xFFFFu; hd[7] = r.w >> 16;
         }
         if (a.norm_mean != nullptr) {  // same for every lane of the launch
           // training-mode batch norm of the column, statistics given:
@@ -240,18 +270,17 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const bool pos = v[k][i] > 0.f;
-          const bool keep = ud[i] > a.p;
-          float r = pos ? v[k][i] : 0.f;
-          r = r * (keep ? 1.f : 0.f);
-          r = r * a.pinv;
-          v[k][i] = r;
+          const bool keep = NOISE_IN ? (ud[i] > a.p) : (hd[i] >= a.act_keep_from);
+          // (r * keep) * pinv of the separate kernel, keep being 1 or 0: r * pinv or r * 0, the same values
+          const float r = pos ? v[k][i] : 0.f;
+          v[k][i] = r * (keep ? a.pinv : 0.f);
           m |= static_cast<uint32_t>(pos && keep) << i;
         }
         // y leaves through LDS: an oct per lane would make every 16-byte store
         // instruction skip every other 16 bytes, which halves the store rate
         ybuf[(k * kBlock + t) * 2 + 0] = f32x4{v[k][0], v[k][1], v[k][2], v[k][3]};
         ybuf[(k * kBlock + t) * 2 + 1] = f32x4{v[k][4], v[k][5], v[k][6], v[k][7]};
-        a.mask_bytes[blk] = static_cast<uint8_t>(m);
+        (a.mask_bytes + row_base * g8)[blk_local] = static_cast<uint8_t>(m);
       }
     }
   }
@@ -267,11 +296,12 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
         const int q = s * kWave + (t & (kWave - 1));
         const int src = wave_first + (q >> 1);  // the thread that produced this quad
         const int half = q & 1;
-        const int64_t n_src = static_cast<int64_t>(blockIdx.x) * rows_per_wg + (src >> a.lpr_log2);
+        const int row_src = src >> a.lpr_log2;
         const int j_src = oct_of(src & (lpr - 1), k);
-        if (n_src < a.N && j_src < a.opr) {
+        if (row_src < rows_here && j_src < a.opr) {
           const f32x4 val = ybuf[(k * kBlock + src) * 2 + half];
-          nt_store4(a.y + n_src * a.G + 8 * j_src + 4 * half, val.x, val.y, val.z, val.w);
+          nt_store4(a.y + row_base * a.G + (static_cast<off_t>(row_src) * G + static_cast<off_t>(8 * j_src + 4 * half)),
+                    val.x, val.y, val.z, val.w);
         }
       }
     }
@@ -302,47 +332,43 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       sc = recip * B;
     }
     if (row_ok && lane_in_row == 0) {
-      if (a.scale_f32) a.scale_f32[n] = sc;
-      if (a.min_f32) a.min_f32[n] = mnv;
-      if (a.scale_bf16) a.scale_bf16[n] = HALF ? half_bits(sc) : f32_to_bf16_rne(sc);
-      if (a.min_bf16) a.min_bf16[n] = HALF ? half_bits(mnv) : f32_to_bf16_rne(mnv);
+      if (a.scale_f32) (a.scale_f32 + row_base)[row_local] = sc;
+      if (a.min_f32) (a.min_f32 + row_base)[row_local] = mnv;
+      if (a.scale_bf16) (a.scale_bf16 + row_base)[row_local] = HALF ? half_bits(sc) : f32_to_bf16_rne(sc);
+      if (a.min_bf16) (a.min_bf16 + row_base)[row_local] = HALF ? half_bits(mnv) : f32_to_bf16_rne(mnv);
     }
   } else {
     if (row_ok) {
-      mnv = a.mn_in[n];
-      sc = a.scale_in[n];
+      mnv = (a.mn_in + row_base)[row_local];
+      sc = (a.scale_in + row_base)[row_local];
     }
   }
 
   // supplied noise: read like x (every lane takes part; rows past the end re-read the last row, their
   // codes are dropped below)
-  float un[(NOISE_IN && !HALF) ? OPT : 1][8];
-  if constexpr (NOISE_IN && !HALF) {
-    if (swz) load_octs_swizzled<OPT>(a.noise + (row_ok ? n : a.N - 1) * a.G + 8 * oct_base, lpr, lane_in_row, un);
-  }
+  float un[(NOISE_IN && swz) ? OPT : 1][8];
+  const float* __restrict__ nw = NOISE_IN ? a.noise + row_base * a.G : nullptr;
+  if constexpr (NOISE_IN && swz) load_octs_swizzled<OPT, off_t>(nw, row_ld_off, lpr, lane_in_row, un);
   uint2 codes[OPT];
 #pragma unroll
   for (int k = 0; k < OPT; ++k) {
     const int j = oct_of(lane_in_row, k);
     float u[8];
     if constexpr (NOISE_IN) {
-      if (swz) {
-        if constexpr (!HALF) {
+      if constexpr (swz) {
 #pragma unroll
-          for (int i = 0; i < 8; ++i) u[i] = un[k][i];
-        }
+        for (int i = 0; i < 8; ++i) u[i] = un[k][i];
       } else if (FULL && !row_ok) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) u[i] = 0.f;
       } else {
-        load_oct<VEC, FULL>(a.noise + row_off + 8 * j, nv[k], u);
+        load_oct<VEC, FULL>(nw + (row_off + static_cast<off_t>(8 * j)), nv[k], u);
       }
     } else {
-      const Philox4 r = philox4x32_10(static_cast<uint32_t>(j), static_cast<uint32_t>(n),
-                                      a.off_lo, a.off_hi, a.seed_lo, a.seed_hi);
+      const Philox4 r = philox4x32_10(static_cast<uint32_t>(j), n_lo, a.off_lo, a.off_hi, a.seed_lo, a.seed_hi);
       philox_uniform8(r, u);
     }
-    uint32_t q[8];
+    uint32_t q[8];  // the code in the low byte
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       // quantization_cuda_kernel.cu:89, one rounding per operation
@@ -351,14 +377,30 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       tq = tq * sc;
       if constexpr (HALF) tq = round_to_half(tq);
       tq = tq + u[i];
-      tq = tq - 0.5f;
-      tq = fmaxf(tq, 0.f);
-      const uint32_t qi = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
-      q[i] = ((FULL ? row_ok : (i < nv[k])) ? qi : 0u) & 0xFFu;
+      if constexpr (FUSED) {
+        // scale and min come from this row: tq < 2^bits + 2
+        q[i] = code_in_low_byte(tq);
+      } else {
+        tq = tq - 0.5f;
+        tq = fmaxf(tq, 0.f);
+        q[i] = float2int_rn_sat(tq);
+      }
+      if constexpr (!FULL) q[i] = (i < nv[k]) ? q[i] : 0u;
     }
-    codes[k] = make_uint2(q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24),
-                          q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24));
-    if constexpr (WPT > 1) stage[k * kBlock + t] = codes[k];
+    codes[k] = make_uint2(low_bytes4(q[0], q[1], q[2], q[3]), low_bytes4(q[4], q[5], q[6], q[7]));
+    if constexpr (FULL) {
+      if (!row_ok) codes[k] = make_uint2(0u, 0u);
+    }
+    if constexpr (WPT == 8) {
+      // one bit per code: every lane moves its row's bits into place first (bits shifted past bit 7 of a byte
+      // vanish, as in the reference's uint8 accumulator), so that the lane that packs only has to OR eight words
+      constexpr uint32_t kByte = 0x01010101u;
+      const int sh = row_local & 7;
+      const uint32_t keep = (0xFFu >> sh) * kByte;
+      stage[k * kBlock + t] = make_uint2((codes[k].x & keep) << sh, (codes[k].y & keep) << sh);
+    } else if constexpr (WPT > 1) {
+      stage[k * kBlock + t] = codes[k];
+    }
   }
   if constexpr (WPT > 1) __syncthreads();  // 8-bit codes: one row per byte, nothing to combine
 
@@ -369,6 +411,14 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
       const int j = oct_of(lane_in_row, k);
       if (j >= a.opr) continue;
       uint32_t w0 = codes[k].x, w1 = codes[k].y;
+      if constexpr (WPT == 8) {
+#pragma unroll
+        for (int i = 1; i < WPT; ++i) {
+          const uint2 s = stage[k * kBlock + t + i * lpr];  // already in place
+          w0 |= s.x;
+          w1 |= s.y;
+        }
+      } else {
 #pragma unroll
       for (int i = 1; i < WPT; ++i) {
         // uint8 accumulator of the reference: bits shifted past bit 7 vanish
@@ -378,8 +428,10 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
         w0 |= (s.x & keep) << (i * BITS);
         w1 |= (s.y & keep) << (i * BITS);
       }
+      }
       const int d0 = 8 * j;
-      uint8_t* dst = a.packed + (n / WPT) * a.G + d0;
+      // row_base is a multiple of 8, hence of WPT
+      uint8_t* dst = a.packed + (row_base / WPT) * a.G + (static_cast<off_t>(row_local / WPT) * G + static_cast<off_t>(d0));
       if (a.out_vec == 8) {
         // one 8-byte store: written as two struct members, the compiler hoists the
         // first word's store out of this branch and issues two 4-byte stores
@@ -478,7 +530,8 @@ static Geometry plan_rows(int64_t G, int max_opt, int opt_hint = 0) {
   g.opt = opt;
   const int octs_per_pass = (1 << l2) * opt;
   g.grid_y = (g.opr + octs_per_pass - 1) / octs_per_pass;
-  g.full = (G % 8 == 0) && (g.opr == octs_per_pass * g.grid_y);
+  // whole rows of whole octs on at least two lanes (the row-contiguous loads pair up neighbouring lanes)
+  g.full = (G % 8 == 0) && (g.opr == octs_per_pass * g.grid_y) && l2 >= 1;
   return g;
 }
 
@@ -750,6 +803,8 @@ static int act_pack_common(const float* x, const float* norm_mean, const float* 
   a.p = p;
   // quantization_cuda_kernel.cu:456: float pinv = 1. / (1. - p), evaluated in double
   a.pinv = static_cast<float>(1.0 / (1.0 - static_cast<double>(p)));
+  // u = (h + 0.5) / 65536 > p  <=>  h > 65536 p - 0.5  <=>  h >= floor(65536 p - 0.5) + 1   (0 <= p < 1, exact in double)
+  a.act_keep_from = static_cast<uint32_t>(static_cast<int>(std::floor(65536.0 * static_cast<double>(p) - 0.5)) + 1);
   a.y = y;
   a.mask_bytes = reinterpret_cast<uint8_t*>(mask);
   a.mask_tail_begin = N * G / 8;

@@ -42,7 +42,6 @@
 namespace exact {
 
 constexpr int kStepFeatures = 16;  // K of one MFMA
-constexpr int kSplitWaves = 4;     // wavefronts of a workgroup that share one 32-row tile
 
 // Eight consecutive floats of a row starting at column `col`, zeros from column
 // `limit` on; VEC = the widest aligned access (limit % VEC == 0, col % VEC == 0).
@@ -121,46 +120,43 @@ __global__ __launch_bounds__(kBlock) void rp_prepare_kernel(const float* __restr
 }
 
 // ---- forward -----------------------------------------------------------------
-// One workgroup per 32 rows; its four wavefronts split the D features between
-// them (whole k-steps, ceil(steps / 4) each) and meet in LDS: part[wave][tile]
-// [register][lane].  A wavefront issues the loads of four k-steps (eight 16-byte
-// loads per lane) and the matching table fragments together.
-template <int VEC, int NT, int BP>
-__device__ __forceinline__ void rp_fwd_partial(const float* __restrict__ X, const u32x4* __restrict__ frags, int64_t N,
-                                               int D, floatx16 (&acc)[NT]) {
+// One wavefront per 32 rows, one wavefront per workgroup: no workgroup barrier
+// anywhere.  The wavefront walks the D features in k-steps of 16, the loads of
+// KS steps issued together (two 16-byte loads per lane and step, the steps'
+// table fragments beside them), and accumulates in step order.  (A workgroup of
+// four wavefronts that split the features and met in LDS was measured against
+// this form: equal at 256 -> 32, 15 % slower at 256 -> 64.)
+// `frags` holds `tiles` column tiles per k-step; the wavefront multiplies by the NT tiles from `tile0` on.
+template <int VEC, int NT, int BP, int KS>
+__device__ __forceinline__ void rp_fwd_rows(const float* __restrict__ X, const u32x4* __restrict__ frags, int64_t N,
+                                            int D, int64_t row0, floatx16 (&acc)[NT], int tiles = NT, int tile0 = 0) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
   const int half = lane >> 5;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTile;
   const int64_t my_row = (row0 + (lane & 31) < N) ? row0 + (lane & 31) : N - 1;
   const float* xrow = X + my_row * D;
   const int total = (D + kStepFeatures - 1) / kStepFeatures;
-  const int per_wave = (total + kSplitWaves - 1) / kSplitWaves;
-  const int first = wave * per_wave;
-  const int last = (first + per_wave < total) ? first + per_wave : total;  // exclusive; may be <= first
-  const int limit = (last * kStepFeatures < D) ? last * kStepFeatures : D;   // my slice ends here (D % VEC == 0)
 
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
 
-  for (int s0 = first; s0 < last; s0 += 4) {
-    float a[4][8];
-    if ((s0 + 4) * kStepFeatures <= limit) {  // wave-uniform: the four steps lie inside my slice, nothing to mask
+  for (int s0 = 0; s0 < total; s0 += KS) {
+    float a[KS][8];
+    if ((s0 + KS) * kStepFeatures <= D) {  // wave-uniform: the KS steps lie inside the row, nothing to mask
 #pragma unroll
-      for (int sb = 0; sb < 4; ++sb) load8<VEC>(xrow, (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb]);
+      for (int sb = 0; sb < KS; ++sb) load8<VEC>(xrow, (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb]);
     } else {
 #pragma unroll
-      for (int sb = 0; sb < 4; ++sb) load8<VEC>(xrow, (s0 + sb) * kStepFeatures + 8 * half, limit, a[sb]);  // zeros past my slice
+      for (int sb = 0; sb < KS; ++sb) load8<VEC>(xrow, (s0 + sb) * kStepFeatures + 8 * half, D, a[sb]);  // zeros past the row
     }
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb) {
-      const int st = (s0 + sb < last) ? s0 + sb : s0;  // a step past my slice meets zeros: any valid fragment will do
+    for (int sb = 0; sb < KS; ++sb) {
+      const int st = (s0 + sb < total) ? s0 + sb : s0;  // a step past the row meets zeros: any valid fragment will do
       const Split8 pieces = split3x8(a[sb]);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const u32x4* src = frags + (static_cast<int64_t>(st) * NT + nt) * BP * kWave + lane;
+        const u32x4* src = frags + (static_cast<int64_t>(st) * tiles + tile0 + nt) * BP * kWave + lane;
         u32x4 b[BP];
 #pragma unroll
         for (int p = 0; p < BP; ++p) b[p] = src[p * kWave];
@@ -170,81 +166,81 @@ __device__ __forceinline__ void rp_fwd_partial(const float* __restrict__ X, cons
   }
 }
 
+// k-steps in flight: four with one column tile (more wavefronts per SIMD do better than more loads per
+// wavefront), eight with several (measured at 256 -> 32 and 256 -> 64)
 template <int NT>
-__device__ __forceinline__ void park_partial(const floatx16 (&acc)[NT], float* part) {
+constexpr int fwd_steps_in_flight() { return NT == 1 ? 4 : 8; }
+
+template <int VEC, int NT, int BP>
+__global__ __launch_bounds__(kWave) void rp_fwd_bf16_kernel(const float* __restrict__ X,
+                                                            const u32x4* __restrict__ table, int64_t N, int D,
+                                                            int k, float* __restrict__ out) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTile;
+  floatx16 acc[NT];
+  rp_fwd_rows<VEC, NT, BP, fwd_steps_in_flight<NT>()>(X, table + 1, N, D, row0, acc);
+  const float c = BP == 1 ? __uint_as_float(table[0][0]) : 1.f;
+  // accumulator register v of lane l is C[8 (v / 4) + 4 (l / 32) + v % 4][l % 32]: a store instruction writes two
+  // rows of 32 consecutive columns
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) part[((wave * NT + nt) * 16 + v) * kWave + lane] = acc[nt][v];
+    for (int v = 0; v < 16; ++v) {
+      const int64_t n = row0 + 8 * (v / 4) + 4 * half + (v % 4);
+      const int col = nt * kTile + l32;
+      if (n < N && col < k) __builtin_nontemporal_store(BP == 1 ? acc[nt][v] * c : acc[nt][v], out + n * k + col);
+    }
 }
 
-template <int VEC, int NT, int BP>
-__global__ __launch_bounds__(kBlock) void rp_fwd_bf16_kernel(const float* __restrict__ X,
-                                                             const u32x4* __restrict__ table, int64_t N, int D,
-                                                             int k, float* __restrict__ out) {
-  HIP_DYNAMIC_SHARED(float, part)  // [4 waves][NT][16][64]
-  floatx16 acc[NT];
-  rp_fwd_partial<VEC, NT, BP>(X, table + 1, N, D, acc);
-  park_partial<NT>(acc, part);
-  __syncthreads();
-  const float c = BP == 1 ? __uint_as_float(table[0][0]) : 1.f;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTile;
-  if (k % 4 == 0 && al16(out)) {
-    // the tile as quads in row-major order: a store instruction covers whole rows
-    const int quads_per_row = k / 4;
-    for (int q = threadIdx.x; q < kTile * quads_per_row; q += kBlock) {
-      const int i = q / quads_per_row, j0 = 4 * (q - i * quads_per_row);
-      const int nt = j0 >> 5, v = 4 * (i >> 3) + (i & 3), ln = (j0 & 31) + 32 * ((i & 7) >> 2);
-      f32x4 s = *reinterpret_cast<const f32x4*>(part + ((0 * NT + nt) * 16 + v) * kWave + ln);
-#pragma unroll
-      for (int w = 1; w < kSplitWaves; ++w) s += *reinterpret_cast<const f32x4*>(part + ((w * NT + nt) * 16 + v) * kWave + ln);
-      if constexpr (BP == 1) s *= c;
-      if (row0 + i < N) __builtin_nontemporal_store(s, reinterpret_cast<f32x4*>(out + (row0 + i) * k + j0));
-    }
-  } else {
-    for (int e = threadIdx.x; e < kTile * k; e += kBlock) {
-      const int i = e / k, j = e - i * k;
-      const int nt = j >> 5, v = 4 * (i >> 3) + (i & 3), ln = (j & 31) + 32 * ((i & 7) >> 2);
-      float s = part[((0 * NT + nt) * 16 + v) * kWave + ln];
-#pragma unroll
-      for (int w = 1; w < kSplitWaves; ++w) s += part[((w * NT + nt) * 16 + v) * kWave + ln];
-      if constexpr (BP == 1) s = s * c;
-      if (row0 + i < N) __builtin_nontemporal_store(s, out + (row0 + i) * k + j);
-    }
-  }
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Projection and quantisation in one launch.  Once the four partial tiles are in
-// LDS the accumulator layout (a lane = one column of the tile) has served its
-// purpose, and the epilogue reads the tile the way the row-wise pack kernel
-// works: a lane owns an "oct" -- eight consecutive columns of one row, the
-// elements of one Philox block (block (d / 8, n) serves columns 8 (d / 8) .. + 7
-// of row n) -- so the row statistics are eight local comparisons and a butterfly
-// over the row's lanes, and no random number is computed twice.  The sums are
-// formed in the order rp_fwd_bf16_kernel forms them and the arithmetic is
-// that of exact_minmax_pack_f32 (quantization_cuda_kernel.cu:89, one rounding
-// per operation), so the bytes equal those of the two launches.  The 8 / bits
-// rows that share a packed byte meet through a second LDS array: every lane
-// parks its row's bits of eight bytes, then one lane per (row group, oct) ORs
-// the group's rows and stores the eight bytes.
+// Projection and quantisation in one launch.  The wavefront turns its finished
+// tile through LDS: out of the accumulator layout (a lane = one column) into the
+// layout the row-wise pack kernel works in, where a lane owns an "oct" -- eight
+// consecutive columns of one row, the elements of one Philox block (block
+// (d / 8, n) serves columns 8 (d / 8) .. + 7 of row n) -- so the row statistics
+// are eight local comparisons and a butterfly over the row's lanes, and no
+// random number is computed twice.  The sums are those of rp_fwd_bf16_kernel
+// (same loop) and the arithmetic is that of exact_minmax_pack_f32
+// (quantization_cuda_kernel.cu:89, one rounding per operation), so the bytes
+// equal those of the two launches.  The 8 / bits rows that share a packed byte
+// meet through a second LDS array: every lane parks its row's bits of eight
+// bytes, then one lane per (row group, oct) ORs the group's rows and stores the
+// eight bytes.  Both arrays are private to the wavefront, whose LDS accesses
+// complete in order: the hand-overs need no workgroup barrier.
 constexpr int kStagePitch = 16;  // octs per row in the hand-over array: k <= 128
+template <int NT>
+constexpr int fwd_tile_pitch() { return NT * kTile + 4; }  // floats per tile row: 16-byte aligned rows, rows 4 apart on other banks
 
 template <int VEC, int NT, int BP, bool NOISE_IN>
-__global__ __launch_bounds__(kBlock) void rp_fwd_pack_bf16_kernel(const RpPackArgs a, const u32x4* __restrict__ table) {
-  // [4 waves][NT][16][64] floats, then uint64 [32 rows][kStagePitch]; at NT == 4 the partial tiles fill the 64 KB a
-  // workgroup may have, and the hand-over array takes their place once every lane has read its sums
-  HIP_DYNAMIC_SHARED(float, part)
+__global__ __launch_bounds__(kWave) void rp_fwd_pack_bf16_kernel(const RpPackArgs a, const u32x4* __restrict__ table) {
+  HIP_DYNAMIC_SHARED(float, tile)  // [32][pitch] floats, then uint64 [32][kStagePitch]
+  constexpr int PITCH = fwd_tile_pitch<NT>();
+  // passes of the 64 lanes over the tile's (row, oct) pairs: 32 rows x (1, 2 or 4 | 8 | 16) lanes per row
+  constexpr int PASSES = NT == 1 ? 2 : (NT == 2 ? 4 : 8);
+  uint64_t* stage = reinterpret_cast<uint64_t*>(tile + kTile * PITCH);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTile;
   {
     floatx16 acc[NT];
-    rp_fwd_partial<VEC, NT, BP>(a.X, table + 1, a.N, a.D, acc);
-    park_partial<NT>(acc, part);
+    rp_fwd_rows<VEC, NT, BP, fwd_steps_in_flight<NT>()>(a.X, table + 1, a.N, a.D, row0, acc);
+    const float c = BP == 1 ? __uint_as_float(table[0][0]) : 1.f;
+    const int half = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        tile[(8 * (v / 4) + 4 * half + (v % 4)) * PITCH + nt * kTile + l32] = BP == 1 ? acc[nt][v] * c : acc[nt][v];
   }
-  __syncthreads();
-  uint64_t* stage = reinterpret_cast<uint64_t*>(NT < 4 ? part + kSplitWaves * NT * 16 * kWave : part);
-  uint64_t parked[2] = {0, 0};  // this lane's words of the (at most two) passes below
-  const float c = BP == 1 ? __uint_as_float(table[0][0]) : 1.f;
+  wave_sync_lds();
+  uint64_t parked[PASSES];  // this lane's words of the passes below
+#pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) parked[pass] = 0;
   const int k = a.k, bits = a.bits;
   const int wpt = 8 / bits;
   const float B = static_cast<float>((1 << bits) - 1);
@@ -252,34 +248,20 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_pack_bf16_kernel(const RpPackAr
   int opr_log = 0;
   while ((1 << opr_log) < octs) ++opr_log;  // lanes per row: the next power of two
   const int opr = 1 << opr_log;
-  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTile;
 
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {  // 32 rows x at most 16 lanes = at most two passes of the 256 threads
-    const int t0 = pass * kBlock;
-    if (t0 >= kTile * opr) break;
-    const int t = t0 + threadIdx.x;
-    if (t - (threadIdx.x & (kWave - 1)) >= kTile * opr) break;
+  for (int pass = 0; pass < PASSES; ++pass) {
+    if (pass * kWave >= kTile * opr) break;
+    const int t = pass * kWave + lane;
     const int i = (t >> opr_log) & (kTile - 1), oct = t & (opr - 1);  // lanes past the tile (k <= 8 only) mirror a real row
     const bool live = t < kTile * opr && oct < octs;
     const int64_t n = row0 + i;
     const int j0 = live ? 8 * oct : 0;
     // ---- the eight sums ------------------------------------------------------
-    const int nt = j0 >> 5, v = 4 * (i >> 3) + (i & 3), ln = (j0 & 31) + 32 * ((i & 7) >> 2);
     float x[8];
     {
-      const float* src = part + ((0 * NT + nt) * 16 + v) * kWave + ln;
-      f32x4 lo4 = *reinterpret_cast<const f32x4*>(src), hi4 = *reinterpret_cast<const f32x4*>(src + 4);
-#pragma unroll
-      for (int w = 1; w < kSplitWaves; ++w) {
-        const float* more = part + ((w * NT + nt) * 16 + v) * kWave + ln;
-        lo4 += *reinterpret_cast<const f32x4*>(more);
-        hi4 += *reinterpret_cast<const f32x4*>(more + 4);
-      }
-      if constexpr (BP == 1) {
-        lo4 *= c;
-        hi4 *= c;
-      }
+      const float* src = tile + i * PITCH + j0;
+      const f32x4 lo4 = *reinterpret_cast<const f32x4*>(src), hi4 = *reinterpret_cast<const f32x4*>(src + 4);
       x[0] = lo4.x; x[1] = lo4.y; x[2] = lo4.z; x[3] = lo4.w; x[4] = hi4.x; x[5] = hi4.y; x[6] = hi4.z; x[7] = hi4.w;
     }
     // ---- row statistics --------------------------------------------------------
@@ -312,31 +294,34 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_pack_bf16_kernel(const RpPackAr
     }
     // ---- quantise; this row's bits of the eight bytes ------------------------------
     const int shift = (i & (wpt - 1)) * bits;
-    uint32_t word[2] = {0u, 0u};
+    uint32_t q[8];  // the code in the low byte
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       float tq = x[e] - mn;
       tq = tq * sc;
       tq = tq + u[e];
-      tq = tq - 0.5f;
-      tq = fmaxf(tq, 0.f);
-      const uint32_t q = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
-      const uint32_t byte = (live && j0 + e < k && n < a.N) ? ((q << shift) & 0xFFu) : 0u;  // uint8_t arithmetic of the reference
-      word[e >> 2] |= byte << (8 * (e & 3));
+      q[e] = code_in_low_byte(tq);  // scale and min are this row's own: tq < 2^bits + 2
     }
+    // uint8_t arithmetic of the reference: bits shifted past bit 7 of a byte vanish; columns past k and rows
+    // past N contribute nothing
+    const uint32_t keep = (0xFFu >> shift) * 0x01010101u;
+    const int cols = (live && n < a.N) ? (k - j0 < 8 ? (k - j0 < 0 ? 0 : k - j0) : 8) : 0;
+    const uint64_t valid = cols >= 8 ? ~uint64_t{0} : ((uint64_t{1} << (8 * cols)) - 1);
+    uint32_t word[2];
+    word[0] = ((low_bytes4(q[0], q[1], q[2], q[3]) & keep) << shift) & static_cast<uint32_t>(valid);
+    word[1] = ((low_bytes4(q[4], q[5], q[6], q[7]) & keep) << shift) & static_cast<uint32_t>(valid >> 32);
     parked[pass] = static_cast<uint64_t>(word[0]) | (static_cast<uint64_t>(word[1]) << 32);
   }
-  if constexpr (NT == 4) __syncthreads();  // the partial tiles have been read: their place is free
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int t = pass * kBlock + threadIdx.x;
+  for (int pass = 0; pass < PASSES; ++pass) {
+    const int t = pass * kWave + lane;
     if (t < kTile * opr) stage[((t >> opr_log) & (kTile - 1)) * kStagePitch + (t & (opr - 1))] = parked[pass];
   }
-  __syncthreads();
+  wave_sync_lds();
   // ---- one lane per (row group, oct): OR the group's rows, store eight bytes -----------
   const int groups = kTile / wpt;
   const bool wide = (k & 7) == 0 && (reinterpret_cast<uintptr_t>(a.packed) & 7u) == 0;
-  for (int t = threadIdx.x; t < groups * octs; t += kBlock) {
+  for (int t = lane; t < groups * octs; t += kWave) {
     const int g = t / octs, oct = t - g * octs;
     if (row0 + static_cast<int64_t>(g) * wpt >= a.N) continue;
     uint64_t w = 0;
@@ -349,7 +334,135 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_pack_bf16_kernel(const RpPackAr
       for (int e = 0; e < cnt; ++e) dst[e] = static_cast<uint8_t>(w >> (8 * e));
     }
   }
-  if (blockIdx.x == 0 && threadIdx.x == 0) a.packed[a.pad_index] = 0;
+  if (blockIdx.x == 0 && lane == 0) a.packed[a.pad_index] = 0;
+}
+
+// ---- tall operand times a small dense matrix ----------------------------------------
+// out[N, K] = X[N, D] . M[D, K] (+ bias[K]) (+ addend[N, K]) for the linear maps of a
+// layer (F.linear and the input gradient of linear_backward, backward_func.cc:83-87):
+// the forward loop above with M split in three (six bf16 products per fp32
+// product, fp32 accuracy), up to eight column tiles per wavefront -- wider
+// matrices take one launch per slab of 256 columns -- and an epilogue that adds
+// a bias row and / or a matrix (which may be `out` itself: every element is read
+// and written by the same lane).  The fragments of M come from
+// exact_tall_gemm_prepare_bf16, which also takes M transposed (a weight as
+// F.linear holds it).  No atomics: the result does not depend on the launch.
+#ifndef EXACT_GEMM_SLAB_TILES
+#define EXACT_GEMM_SLAB_TILES 4
+#endif
+#ifndef EXACT_GEMM_ROW_TILES
+#define EXACT_GEMM_ROW_TILES 1
+#endif
+#ifndef EXACT_GEMM_STEPS
+#define EXACT_GEMM_STEPS 4
+#endif
+constexpr int kGemmSlabTiles = EXACT_GEMM_SLAB_TILES;  // column tiles (of 32) one launch covers, at most 8
+constexpr int kGemmRowTiles = EXACT_GEMM_ROW_TILES;    // row tiles (of 32) per wavefront
+constexpr int kGemmSteps = EXACT_GEMM_STEPS;           // k-steps whose loads are issued together
+
+__global__ __launch_bounds__(kBlock) void gemm_prepare_kernel(const float* __restrict__ M, int64_t ld, int transposed,
+                                                              int D, int K, u32x4* __restrict__ table) {
+  const TableShape ts = table_shape(D, K, 3);
+  const int64_t frags = static_cast<int64_t>(ts.steps_d) * ts.tiles_k * kWave;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx == 0) {
+    u32x4 head = {0u, 0u, 0u, 0u};
+    table[0] = head;
+  }
+  if (idx >= frags) return;
+  const int l = static_cast<int>(idx & (kWave - 1));
+  const int tile = static_cast<int>((idx / kWave) % ts.tiles_k), step = static_cast<int>(idx / (static_cast<int64_t>(kWave) * ts.tiles_k));
+  float r[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int d = step * kStepFeatures + 8 * (l >> 5) + i, c = tile * kTile + (l & 31);
+    const bool inside = d < D && c < K;
+    r[i] = inside ? (transposed ? M[static_cast<int64_t>(c) * ld + d] : M[static_cast<int64_t>(d) * ld + c]) : 0.f;
+  }
+  u32x4* dst = table + 1 + (static_cast<int64_t>(step) * ts.tiles_k + tile) * 3 * kWave + l;
+  const Split8 s = split3x8(r);
+  dst[0] = s.hi;
+  dst[kWave] = s.mid;
+  dst[2 * kWave] = s.lo;
+}
+
+// A wavefront owns RT row tiles (32 RT rows) and NT column tiles, with the loads of KS k-steps of X in flight.
+// Measured on [169343 .. 2449029, 100 .. 604] x [.., 40 .. 352]: one row tile, four column tiles and four steps
+// is the fastest split (two or three row tiles per wavefront -- every fragment of M then serves several
+// products -- cost more in occupancy than they save in fragment loads: 330 against 236 us at 256 x 256).  The
+// kernel then equals the framework's fp32 GEMM at 256 output columns and beats it by 20 - 25 % at 40 - 47.
+template <int RT, int NT, int KS>
+__global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __restrict__ X,
+                                                               const u32x4* __restrict__ table, int64_t N, int D, int K,
+                                                               int tiles, int tile0, const float* __restrict__ bias,
+                                                               const float* addend, int64_t ldc, float* out,
+                                                               int64_t ldo) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int half = lane >> 5, l32 = lane & 31;
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * (kTile * RT);
+  const u32x4* frags = table + 1;
+  const float* xrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int64_t r = row0 + rt * kTile + l32;
+    xrow[rt] = X + (r < N ? r : N - 1) * D;
+  }
+  const int total = (D + kStepFeatures - 1) / kStepFeatures;
+  floatx16 acc[RT][NT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[rt][nt][v] = 0.f;
+
+  for (int s0 = 0; s0 < total; s0 += KS) {
+    float a[KS][RT][8];
+    if ((s0 + KS) * kStepFeatures <= D) {  // wave-uniform: the KS steps lie inside the row, nothing to mask
+#pragma unroll
+      for (int sb = 0; sb < KS; ++sb)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb][rt]);
+    } else {
+#pragma unroll
+      for (int sb = 0; sb < KS; ++sb)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, D, a[sb][rt]);
+    }
+#pragma unroll
+    for (int sb = 0; sb < KS; ++sb) {
+      const int st = (s0 + sb < total) ? s0 + sb : s0;  // a step past the row meets zeros: any valid fragment will do
+      Split8 pieces[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) pieces[rt] = split3x8(a[sb][rt]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const u32x4* src = frags + (static_cast<int64_t>(st) * tiles + tile0 + nt) * 3 * kWave + lane;
+        u32x4 b[3];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) b[p] = src[p * kWave];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[rt][nt] = step_product<3>(pieces[rt], b, acc[rt][nt]);
+      }
+    }
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int col = (tile0 + nt) * kTile + l32;
+    const float b = (bias != nullptr && col < K) ? bias[col] : 0.f;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t n = row0 + rt * kTile + 8 * (v / 4) + 4 * half + (v % 4);
+        if (n < N && col < K) {
+          float val = acc[rt][nt][v];
+          if (bias != nullptr) val = val + b;
+          if (addend != nullptr) val = val + addend[n * ldc + col];
+          __builtin_nontemporal_store(val, out + n * ldo + col);
+        }
+      }
+  }
 }
 
 // ---- backward ----------------------------------------------------------------
@@ -364,12 +477,6 @@ __global__ __launch_bounds__(kBlock) void rp_fwd_pack_bf16_kernel(const RpPackAr
 // hand-over inside it needs no workgroup barrier.
 template <int NT>
 constexpr int bwd_tile_pitch() { return NT * kTile + 8; }  // 4 * pitch = 32 (mod 64): the two half-waves hit different banks
-
-__device__ __forceinline__ void wave_sync_lds() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 
 template <int VEC, int NT, int BP, int KS, bool STAGED>  // KS: k-steps whose loads are issued (2, 4 or 8 >= the steps of k)
 __global__ __launch_bounds__(kBlock) void rp_bwd_bf16_kernel(const float* __restrict__ Xr,
@@ -465,18 +572,16 @@ __global__ __launch_bounds__(kBlock) void rp_bwd_bf16_kernel(const float* __rest
 
 // ---- launches ----------------------------------------------------------------
 template <int NT>
-constexpr size_t fwd_lds_bytes() { return static_cast<size_t>(kSplitWaves) * NT * 16 * kWave * sizeof(float); }
-template <int NT>
-constexpr size_t fwd_pack_lds_bytes() { return fwd_lds_bytes<NT>() + (NT < 4 ? kTile * kStagePitch * sizeof(uint64_t) : 0); }
+constexpr size_t fwd_pack_lds_bytes() { return sizeof(float) * kTile * fwd_tile_pitch<NT>() + sizeof(uint64_t) * kTile * kStagePitch; }
 
 template <int VEC, int BP>
 static int rp_fwd_bf16_launch(const float* X, const u32x4* table, int64_t N, int D, int k, float* out, hipStream_t s) {
-  const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile)), block(kBlock);
+  const dim3 grid(static_cast<unsigned>((N + kTile - 1) / kTile)), block(kWave);
   switch ((k + kTile - 1) / kTile) {
-    case 1: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 1, BP>), grid, block, fwd_lds_bytes<1>(), s, X, table, N, D, k, out); break;
-    case 2: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 2, BP>), grid, block, fwd_lds_bytes<2>(), s, X, table, N, D, k, out); break;
-    case 3: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 3, BP>), grid, block, fwd_lds_bytes<3>(), s, X, table, N, D, k, out); break;
-    case 4: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 4, BP>), grid, block, fwd_lds_bytes<4>(), s, X, table, N, D, k, out); break;
+    case 1: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 1, BP>), grid, block, 0, s, X, table, N, D, k, out); break;
+    case 2: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 2, BP>), grid, block, 0, s, X, table, N, D, k, out); break;
+    case 3: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 3, BP>), grid, block, 0, s, X, table, N, D, k, out); break;
+    case 4: hipLaunchKernelGGL((rp_fwd_bf16_kernel<VEC, 4, BP>), grid, block, 0, s, X, table, N, D, k, out); break;
     default: return EXACT_E_SHAPE;
   }
   return launch_status();
@@ -484,7 +589,7 @@ static int rp_fwd_bf16_launch(const float* X, const u32x4* table, int64_t N, int
 
 template <int VEC, int BP, bool NOISE_IN>
 static int rp_fwd_pack_bf16_launch(const RpPackArgs& a, const u32x4* table, hipStream_t s) {
-  const dim3 grid(static_cast<unsigned>((a.N + kTile - 1) / kTile)), block(kBlock);
+  const dim3 grid(static_cast<unsigned>((a.N + kTile - 1) / kTile)), block(kWave);
   switch ((a.k + kTile - 1) / kTile) {
     case 1: hipLaunchKernelGGL((rp_fwd_pack_bf16_kernel<VEC, 1, BP, NOISE_IN>), grid, block, fwd_pack_lds_bytes<1>(), s, a, table); break;
     case 2: hipLaunchKernelGGL((rp_fwd_pack_bf16_kernel<VEC, 2, BP, NOISE_IN>), grid, block, fwd_pack_lds_bytes<2>(), s, a, table); break;
@@ -634,6 +739,60 @@ int exact_rp_bwd_bf16_f32(const float* Xr, const void* table, int64_t N, int64_t
   if (k % 2 == 0 && al8(Xr)) return EXACT_RP_GO(2);
   return EXACT_RP_GO(1);
 #undef EXACT_RP_GO
+}
+
+int64_t exact_tall_gemm_table_nbytes(int64_t D, int64_t K) {
+  if (D <= 0 || K <= 0 || D > 4096 || K > 4096) return 0;
+  const TableShape ts = table_shape(static_cast<int>(D), static_cast<int>(K), 3);
+  return 16 * (1 + ts.fwd_units());
+}
+
+int exact_tall_gemm_prepare_bf16(const float* M, int64_t ld, int transposed, int64_t D, int64_t K, void* table,
+                                 void* stream) {
+  if (D <= 0 || K <= 0 || D > 4096 || K > 4096) return EXACT_E_SHAPE;
+  if (transposed != 0 && transposed != 1) return EXACT_E_ARG;
+  if (ld < (transposed ? D : K)) return EXACT_E_SHAPE;
+  if (!M || !table) return EXACT_E_NULL;
+  if (!al16(table)) return EXACT_E_ALIGN;
+  const TableShape ts = table_shape(static_cast<int>(D), static_cast<int>(K), 3);
+  const int64_t frags = ts.fwd_units() / 3;
+  const dim3 grid(static_cast<unsigned>((frags + kBlock - 1) / kBlock)), block(kBlock);
+  hipLaunchKernelGGL(gemm_prepare_kernel, grid, block, 0, static_cast<hipStream_t>(stream), M, ld, transposed,
+                     static_cast<int>(D), static_cast<int>(K), static_cast<u32x4*>(table));
+  return launch_status();
+}
+
+int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64_t D, int64_t K, const float* bias,
+                             const float* addend, int64_t ldc, float* out, int64_t ldo, void* stream) {
+  if (N < 0 || D <= 0 || K <= 0 || D > 4096 || K > 4096 || D % 4 != 0) return EXACT_E_SHAPE;
+  if (ldo < K || (addend && ldc < K)) return EXACT_E_SHAPE;
+  if (N == 0) return EXACT_OK;
+  if (!X || !table || !out) return EXACT_E_NULL;
+  if (!al16(table) || !al16(X)) return EXACT_E_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const u32x4* t = static_cast<const u32x4*>(table);
+  const int d = static_cast<int>(D), kk = static_cast<int>(K);
+  const int tiles = (kk + kTile - 1) / kTile;
+  const int64_t rows_per_wave = static_cast<int64_t>(kTile) * kGemmRowTiles;
+  const dim3 grid(static_cast<unsigned>((N + rows_per_wave - 1) / rows_per_wave)), block(kWave);
+  for (int tile0 = 0; tile0 < tiles; tile0 += kGemmSlabTiles) {
+    const int nt = tiles - tile0 < kGemmSlabTiles ? tiles - tile0 : kGemmSlabTiles;
+#define EXACT_GEMM_GO(NTV)                                                                                          \
+  hipLaunchKernelGGL((tall_gemm_bf16_kernel<kGemmRowTiles, (NTV <= kGemmSlabTiles ? NTV : 1), kGemmSteps>), grid, block, 0, s, X, t, N, \
+                     d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
+    switch (nt) {
+      case 1: EXACT_GEMM_GO(1); break;
+      case 2: EXACT_GEMM_GO(2); break;
+      case 3: EXACT_GEMM_GO(3); break;
+      case 4: EXACT_GEMM_GO(4); break;
+      case 5: EXACT_GEMM_GO(5); break;
+      case 6: EXACT_GEMM_GO(6); break;
+      case 7: EXACT_GEMM_GO(7); break;
+      default: EXACT_GEMM_GO(8); break;
+    }
+#undef EXACT_GEMM_GO
+  }
+  return launch_status();
 }
 
 }  // extern "C"

@@ -121,9 +121,7 @@ __device__ __forceinline__ void rp_quantise_and_pack(const RpPackArgs& a, const 
         float tq = acc[nt][4 * vg + r] - mnv[r];
         tq = tq * sc[r];
         tq = tq + u[r];
-        tq = tq - 0.5f;
-        tq = fmaxf(tq, 0.f);
-        const uint32_t qi = static_cast<uint32_t>(static_cast<int>(rintf(tq)));
+        const uint32_t qi = code_in_low_byte(tq);  // scale and min are this row's own: tq < 2^bits + 2
         q[r] = (col_ok && rbase + r < a.N) ? (qi & 0xFFu) : 0u;
       }
       // ---- pack: byte (n / wpt) * k + d holds rows n .. n + wpt - 1 of column d ----

@@ -275,6 +275,8 @@ class qlinear(Function):
             kept = CompressedActivation.adopt(input, quantized, randmat, project=rp)
         empty_cache(config.empty_cache_threshold)
         ctx.kept, ctx.weight, ctx.bias = kept, weight, bias
+        if input.dim() == 2:
+            return ext_backward_func.tall_matmul(input, weight, transposed=True, bias=bias)
         return F.linear(input, weight, bias)
 
     @staticmethod
@@ -289,7 +291,7 @@ class qlinear(Function):
             # the reference (ops.py:163-165) is never formed; only the order in
             # which fp32 sums are taken differs.
             x_r = dequantize_activation(kept.quantized, kept.stored_shape)
-            grad_input = grad_output.mm(ctx.weight) if ctx.needs_input_grad[0] else None
+            grad_input = ext_backward_func.tall_matmul(grad_output, ctx.weight) if ctx.needs_input_grad[0] else None
             grad_weight = ext_backward_func.weight_gradient(grad_output, x_r).mm(kept.randmat.t())
             grads = (grad_input, grad_weight,
                      ext_backward_func.column_sums(grad_output) if ctx.bias is not None else None)
@@ -450,17 +452,15 @@ class qsage(Function):
             both = x.new_zeros((cin, (width + 31) // 32 * 32))
             both[:, :k] = rand_matrix
             both[:, k:width] = weight_l.detach().t()
-            aggregated = spmm.spmm_csr(rowptr, col, value, x.mm(both)[:, :width + (width & 1)], reduce)
+            aggregated = spmm.spmm_csr(rowptr, col, value, ext_backward_func.tall_matmul(x, both)[:, :width + (width & 1)], reduce)
             quantized = quantize_activation(aggregated[:, :k].contiguous(), None)
             kept_l = CompressedActivation(quantized, rand_matrix, x.shape, torch.Size((n, k)))
-            out = torch.addmm(aggregated[:, k:width], x, weight_r.t())
-            if bias_l is not None:
-                out += bias_l
+            out = ext_backward_func.tall_matmul(x, weight_r, transposed=True, bias=bias_l, addend=aggregated[:, k:width])
         else:
             aggregated = spmm.spmm_csr(rowptr, col, value, x, reduce)
             kept_l = CompressedActivation.compress(aggregated, scheme_l)
-            out = aggregated.mm(weight_l.t()) if bias_l is None else torch.addmm(bias_l, aggregated, weight_l.t())
-            out.addmm_(x, weight_r.t())
+            out = ext_backward_func.tall_matmul(aggregated, weight_l, transposed=True, bias=bias_l)
+            ext_backward_func.tall_matmul(x, weight_r, transposed=True, addend=out, into=out)
         del aggregated
         empty_cache(config.empty_cache_threshold)
         ctx.kept = (kept_l, shared)
@@ -486,10 +486,10 @@ class qsage(Function):
         if ctx.needs_input_grad[0]:
             cout, cin = weight_l.shape
             if config.sage_reassociate_backward and cout < cin:
-                grad_x = transpose_product(grad_output).mm(weight_l)
+                grad_x = ext_backward_func.tall_matmul(transpose_product(grad_output), weight_l)
             else:
-                grad_x = transpose_product(grad_output.mm(weight_l))
-            grad_x.addmm_(grad_output, weight_r)
+                grad_x = transpose_product(ext_backward_func.tall_matmul(grad_output, weight_l))
+            ext_backward_func.tall_matmul(grad_output, weight_r, addend=grad_x, into=grad_x)
         grad_wl = _restored_weight_gradient(grad_output, kept_l) if ctx.needs_input_grad[1] else None
         del kept_l
         grad_wr = _restored_weight_gradient(grad_output, shared) if ctx.needs_input_grad[3] else None
@@ -525,10 +525,10 @@ class qgcn(Function):
         cout, cin = weight.shape
         if config.gcn_aggregate_narrow and cin < cout:
             aggregated = spmm.spmm_csr(rowptr, col, value, x, reduce)
-            out = aggregated.mm(weight.t()) if bias is None else torch.addmm(bias, aggregated, weight.t())
+            out = ext_backward_func.tall_matmul(aggregated, weight, transposed=True, bias=bias)
             del aggregated
         else:
-            out = spmm.spmm_csr(rowptr, col, value, x.mm(weight.t()), reduce)
+            out = spmm.spmm_csr(rowptr, col, value, ext_backward_func.tall_matmul(x, weight, transposed=True), reduce)
             if bias is not None:
                 out += bias
         empty_cache(config.empty_cache_threshold)
@@ -559,7 +559,7 @@ class qgcn(Function):
                 g = spmm.spmm_mean_bw(row, rowptr, col, value, rowcount, colptr, csr2csc, None, grad_output, has_value,
                                       False, True)[1]
             if ctx.needs_input_grad[0]:
-                grad_x = g.mm(weight)
+                grad_x = ext_backward_func.tall_matmul(g, weight)
             if ctx.needs_input_grad[1]:
                 grad_w = _restored_weight_gradient(g, kept)
         del kept

@@ -363,6 +363,30 @@ int exact_rp_minmax_pack_bf16_f32(const float *X, const void *table, int mode, c
                                   int bits, uint8_t *packed, float *scale_f32, float *min_f32,
                                   uint16_t *scale_bf16, uint16_t *min_bf16, void *stream);
 
+/* The dense products of a layer around the compressed activation: out[N, K] =
+ * X[N, D] . M[D, K] (+ bias[K]) (+ addend[N, K]), row-major fp32, N >> D, K.
+ * Replaces `F.linear(input, weight, bias)` of qlinear.forward (ops.py:150) with
+ * M = weight^T, and `grad_output.mm(weight)` of linear_backward
+ * (backward_func.cc:85-86) with M = weight, by the forward projection kernel
+ * above in its any-matrix form: M is split without error into three bf16
+ * matrices and six bf16 matrix-core products stand for each fp32 product (the
+ * neglected ones are below 2^-24 of it), accumulated in fp32.  No atomics: the
+ * result is reproducible.
+ * exact_tall_gemm_prepare_bf16 writes the operand fragments of M into `table`
+ * (exact_tall_gemm_table_nbytes(D, K) bytes, 16-byte aligned, owned by the
+ * caller, valid while M is unchanged); M has row stride `ld` elements and is
+ * read as M[d * ld + c], or as M[c * ld + d] when `transposed` is 1 (a weight
+ * [K, D] as F.linear holds it).
+ * exact_tall_gemm_bf16_f32: X contiguous [N, D], 16-byte aligned, D % 4 == 0,
+ * D and K at most 4096; `bias` and `addend` may be NULL; `addend` (row stride
+ * ldc) may be `out` itself (row stride ldo >= K): out += X . M. */
+int64_t exact_tall_gemm_table_nbytes(int64_t D, int64_t K);
+int exact_tall_gemm_prepare_bf16(const float *M, int64_t ld, int transposed, int64_t D, int64_t K,
+                                 void *table, void *stream);
+int exact_tall_gemm_bf16_f32(const float *X, const void *table, int64_t N, int64_t D, int64_t K,
+                             const float *bias, const float *addend, int64_t ldc, float *out,
+                             int64_t ldo, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

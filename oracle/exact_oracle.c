@@ -52,6 +52,10 @@ void oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t
   philox4x32_10(out, key[0], key[1]);
 }
 
+/* __float2int_rn = cvt.rni.s32.f32: round half to even, clamped to the int32 range (NaN does not reach it:
+ * the fmaxf ahead of it returns 0). */
+static inline int32_t float2int_rn(float t) { return t >= 2147483648.0f ? INT32_MAX : (int32_t)rintf(t); }
+
 static inline float u16_to_uniform(uint32_t h) { return ((float)h + 0.5f) * 0x1p-16f; }
 
 /* noise of element (n, d): counter (d / 8, n, offset_lo, offset_hi), key = seed */
@@ -124,8 +128,8 @@ void oracle_pack(const float *x, const float *mn, const float *scale, const floa
           t = t + u[i];
           t = t - 0.5f;
           t = fmaxf(t, 0.0f);
-          const int32_t val = (int32_t)rintf(t); /* __float2int_rn */
-          local[i] |= (uint8_t)(val << (ni * bits));
+          const int32_t val = float2int_rn(t);
+          local[i] |= (uint8_t)((uint32_t)val << (ni * bits));
         }
       }
       for (int i = 0; i < cnt; ++i) packed[no * G + d0 + i] = local[i];

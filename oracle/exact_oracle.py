@@ -141,7 +141,7 @@ def compute_scale(mn: np.ndarray, mx: np.ndarray, bits: int) -> np.ndarray:
     """`python_int / tensor` is Tensor.__rtruediv__, which torch defines as
     `tensor.reciprocal() * python_int`: TWO fp32 roundings (1/range, then * B),
     not one division.  Pinned by test_oracle.py against torch on the CPU."""
-    with np.errstate(divide="ignore", invalid="ignore"):
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
         recip = (F32(1.0) / (mx.astype(F32) - mn.astype(F32))).astype(F32)
         return (recip * F32(2 ** bits - 1)).astype(F32)
 
@@ -170,7 +170,10 @@ def quantize_values(x, mn, scale, noise) -> np.ndarray:
         t = (t + np.asarray(noise, dtype=F32)).astype(F32)
         t = (t - F32(0.5)).astype(F32)
         t = np.fmax(t, F32(0.0))          # IEEE fmax: NaN -> 0
-        return np.rint(t).astype(np.int32)  # round half to even, like cvt.rni
+        # round half to even, like cvt.rni.s32.f32, which clamps to the int32 range: +inf (a row whose
+        # spread is so small that its reciprocal overflows) gives INT_MAX
+        big = t >= F32(2147483648.0)
+        return np.where(big, np.int32(2147483647), np.rint(np.where(big, F32(0.0), t)).astype(np.int32)).astype(np.int32)
 
 
 def pack_single_precision(x, mn, scale, bits: int, noise) -> np.ndarray:

@@ -45,7 +45,8 @@ def quantize_activation(x, bits, noise):
         t = h(h(xf - mn[:, None]) * scale[:, None])
         t = (t + np.asarray(noise, F32)).astype(F32)
         t = (t - F32(0.5)).astype(F32)
-        q = np.rint(np.fmax(t, F32(0.0))).astype(np.int64)
+        t = np.fmax(t, F32(0.0))
+        q = np.where(t >= F32(2147483648.0), 2147483647, np.rint(np.where(np.isinf(t), F32(0.0), t))).astype(np.int64)   # cvt.rni.s32.f32 saturates
     N, G = x.shape
     wpt = 8 // bits
     n_round = N + (wpt - N % wpt) % wpt

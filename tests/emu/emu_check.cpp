@@ -538,6 +538,61 @@ static void check_dw(int64_t N, int64_t K, int64_t D, int64_t pad, std::mt19937&
   }
 }
 
+// exact_tall_gemm_bf16_f32 on exactly sized buffers: small integers, so the result is the integer product
+// bit for bit; the matrix direct with a row stride and transposed; bias, addend and in-place accumulation.
+static void check_gemm(int64_t N, int64_t D, int64_t K, int64_t pad, std::mt19937& rng) {
+  std::uniform_int_distribution<int> id(-5, 5);
+  const int64_t ld = K + pad, ldt = D + pad, ldc = K + 2 * pad, ldo = K + pad;
+  Buf<float> X(static_cast<size_t>(N * D)), M(static_cast<size_t>(D * ld)), Mt(static_cast<size_t>(K * ldt)), bias(static_cast<size_t>(K)),
+      add(static_cast<size_t>(N * ldc)), out(static_cast<size_t>(N * ldo));
+  for (int64_t i = 0; i < N * D; ++i) X[i] = static_cast<float>(id(rng));
+  for (int64_t i = 0; i < D * ld; ++i) M[i] = static_cast<float>(id(rng));
+  for (int64_t c = 0; c < K; ++c)
+    for (int64_t d = 0; d < ldt; ++d) Mt[c * ldt + d] = d < D ? M[d * ld + c] : 99.f;
+  for (int64_t i = 0; i < K; ++i) bias[i] = static_cast<float>(id(rng));
+  for (int64_t i = 0; i < N * ldc; ++i) add[i] = static_cast<float>(id(rng));
+  const int64_t tbytes = exact_tall_gemm_table_nbytes(D, K);
+  CHECK(tbytes > 0 && tbytes % 16 == 0, "gemm table size");
+  Buf<uint32_t> table(tbytes / 4);
+  for (int variant = 0; variant < 4; ++variant) {
+    const bool transposed = variant & 1;
+    CHECK(exact_tall_gemm_prepare_bf16(transposed ? Mt.p : M.p, transposed ? ldt : ld, transposed, D, K, table.p, nullptr) == 0,
+          "gemm prepare rc");
+    const bool with_bias = variant >= 1, with_add = variant >= 2, in_place = variant == 3;
+    for (int64_t i = 0; i < N * ldo; ++i) out[i] = -777.f;
+    if (in_place)
+      for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < K; ++c) out[n * ldo + c] = add[n * ldc + c];
+    const int rc = exact_tall_gemm_bf16_f32(X.p, table.p, N, D, K, with_bias ? bias.p : nullptr,
+                                            with_add ? (in_place ? out.p : add.p) : nullptr, in_place ? ldo : ldc, out.p, ldo, nullptr);
+    CHECK(rc == 0, "gemm rc %d", rc);
+    for (int64_t n = 0; n < N; ++n)
+      for (int64_t c = 0; c < ldo; ++c) {
+        if (c >= K) {
+          CHECK(out[n * ldo + c] == -777.f, "gemm wrote into the row padding at (%lld, %lld)", (long long)n, (long long)c);
+          continue;
+        }
+        double want = 0;
+        for (int64_t d = 0; d < D; ++d) want += static_cast<double>(X[n * D + d]) * M[d * ld + c];
+        if (with_bias) want += bias[c];
+        if (with_add) want += add[n * ldc + c];
+        CHECK(out[n * ldo + c] == static_cast<float>(want), "gemm variant %d N=%lld D=%lld K=%lld at (%lld, %lld)", variant,
+              (long long)N, (long long)D, (long long)K, (long long)n, (long long)c);
+      }
+  }
+}
+
+static void check_gemm_shapes(std::mt19937& rng) {
+  check_gemm(1, 4, 1, 0, rng);
+  check_gemm(33, 8, 5, 3, rng);
+  check_gemm(70, 256, 256, 0, rng);
+  check_gemm(40, 128, 40, 1, rng);
+  check_gemm(65, 100, 47, 2, rng);
+  check_gemm(31, 604, 332, 0, rng);
+  check_gemm(64, 256, 300, 4, rng);
+  check_gemm(97, 48, 257, 0, rng);
+}
+
 static const int64_t kRpShapes[][3] = {{1, 256, 32}, {31, 256, 32}, {200, 256, 32}, {130, 602, 76}, {140, 100, 25}, {129, 256, 64},
                                        {64, 128, 64}, {77, 50, 15}, {130, 7, 4}, {100, 256, 126}, {33, 256, 128}, {70, 96, 96},
                                        {133, 97, 13}, {260, 1024, 32}, {2000, 256, 32}, {1700, 100, 25},
@@ -560,6 +615,11 @@ int main(int argc, char** argv) {
       check_unpack_only(131077, 8, bits, rng);
     }
     std::printf("unpack sizes ok (failures so far %d)\n", g_fail);
+    return g_fail != 0;
+  }
+  if (mode == "gemm") {  // the tall-operand GEMM only
+    check_gemm_shapes(rng);
+    std::printf("gemm shapes ok (failures so far %d)\n", g_fail);
     return g_fail != 0;
   }
   if (mode == "dw") {  // the weight-gradient kernels only
@@ -620,6 +680,8 @@ int main(int argc, char** argv) {
                            {600, 130, 70, 0}, {513, 32, 200, 5}};
   for (auto& d : ds) check_dw(d[0], d[1], d[2], d[3], rng);
   std::printf("weight gradient ok (failures so far %d)\n", g_fail);
+  check_gemm_shapes(rng);
+  std::printf("tall gemm ok (failures so far %d)\n", g_fail);
   if (mode == "large" || mode == "full") {
     // a line after every group: this part runs for hours under the sanitizer
     for (int bits : {1, 2, 4, 8}) check_quant(20011, 256, bits, bits == 4, rng);

@@ -366,6 +366,32 @@ inline int update_dpp_i32(int v, int ctrl, int row_mask, int bank_mask, bool bou
 inline float update_dpp_any(float v, int c, int rm, int bm, bool bc) { return update_dpp_f32(v, c, rm, bm, bc); }
 inline int update_dpp_any(int v, int c, int rm, int bm, bool bc) { return update_dpp_i32(v, c, rm, bm, bc); }
 
+// v_med3_f32: the median; with a NaN among the operands, v_min3_f32 of them
+// (each v_min_f32 step returns the operand that is not a NaN)
+inline float fmed3(float a, float b, float c) {
+  if (std::isnan(a) || std::isnan(b) || std::isnan(c)) return std::fmin(std::fmin(a, b), c);
+  const float hi = std::fmax(std::fmax(a, b), c);
+  if (hi == a) return std::fmax(b, c);
+  if (hi == b) return std::fmax(a, c);
+  return std::fmax(a, b);
+}
+
+// v_perm_b32: byte i of the result is byte sel[i] of the eight bytes {hi, lo}
+// (0..3 = lo, 4..7 = hi); 8..11 replicate a sign bit, 12 gives 0x00, above 0xFF
+inline uint32_t byte_perm(uint32_t hi, uint32_t lo, uint32_t sel) {
+  const uint64_t pool = (static_cast<uint64_t>(hi) << 32) | lo;
+  uint32_t out = 0;
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t s = (sel >> (8 * i)) & 0xFFu;
+    uint32_t byte;
+    if (s < 8) byte = static_cast<uint32_t>(pool >> (8 * s)) & 0xFFu;
+    else if (s < 12) byte = ((pool >> (16 * (s - 8) + 15)) & 1u) ? 0xFFu : 0u;
+    else byte = s == 12 ? 0u : 0xFFu;
+    out |= byte << (8 * i);
+  }
+  return out;
+}
+
 // v_bitop3_b32: bit i of the result = truth table bit ((a_i << 2) | (b_i << 1) | c_i)
 inline uint32_t bitop3(uint32_t a, uint32_t b, uint32_t c, int table) {
   uint32_t out = 0;
@@ -503,6 +529,8 @@ static inline uint64_t __ballot(bool p) { return hipemu::ballot(p); }
 #define __builtin_amdgcn_mov_dpp(v, ctrl, rm, bm, bc) hipemu::mov_dpp((v), (ctrl), (rm), (bm), (bc))
 #define __builtin_amdgcn_update_dpp(old, v, ctrl, rm, bm, bc) hipemu::update_dpp_any((v), (ctrl), (rm), (bm), (bc))
 #define __builtin_amdgcn_bitop3_b32(a, b, c, table) hipemu::bitop3((a), (b), (c), (table))
+#define __builtin_amdgcn_perm(hi, lo, sel) hipemu::byte_perm((hi), (lo), (sel))
+#define __builtin_amdgcn_fmed3f(a, b, c) hipemu::fmed3((a), (b), (c))
 #define __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, x, y, z) hipemu::mfma_f32_32x32x2f32((a), (b), (c), (x), (y), (z))
 // every active lane of the wavefront arrives before any goes on (a scheduling barrier on the hardware, where the
 // lanes of a wavefront move in lockstep anyway; here the lanes are fibres and must really wait)

@@ -467,6 +467,40 @@ def linear_dw(dy, x, ldy=None, ldx=None, guard=8, expect_rc=0, bf16=False):
     return out[:K * D].reshape(K, D)
 
 
+def tall_gemm(X, M, bias=None, addend=None, transposed=False, ld=None, in_place=False, guard=16, expect_rc=0):
+    """exact_tall_gemm_prepare_bf16 + exact_tall_gemm_bf16_f32: X [N, D] . M [D, K] (+ bias) (+ addend) -> fp32 [N, K].
+    `M` is given as the [D, K] matrix; transposed=True hands it over as its [K, D] transpose, `ld` as a wider row
+    stride with NaN in the padding; in_place=True passes the output (pre-filled with addend) as the addend."""
+    X, M = f32(X), f32(M)
+    N, D = X.shape
+    K = M.shape[1]
+    src = np.ascontiguousarray(M.T) if transposed else M
+    if ld:
+        wide = np.full((src.shape[0], ld), np.float32(np.nan), np.float32); wide[:, :src.shape[1]] = src; src = wide
+    nb = int(emu().exact_tall_gemm_table_nbytes(D, K))
+    assert nb > 0 and nb % 16 == 0
+    raw = np.full(nb + 64 + 16, 0xC3, np.uint8)
+    off = (-raw.ctypes.data) % 16
+    table = raw[off:off + nb + 64]
+    rc = emu().exact_tall_gemm_prepare_bf16(p(src), src.shape[1], int(transposed), D, K, p(table), None)
+    assert rc == 0, rc
+    assert (table[nb:] == 0xC3).all()
+    out = np.full(N * K + guard, np.float32(-777.0), np.float32)
+    b = None if bias is None else f32(bias)
+    a = None if addend is None else f32(addend)
+    if in_place and a is not None:
+        out[:N * K] = a.reshape(-1)
+        rc = emu().exact_tall_gemm_bf16_f32(p(X), p(table), N, D, K, p(b) if b is not None else None, p(out), K, p(out), K, None)
+    else:
+        rc = emu().exact_tall_gemm_bf16_f32(p(X), p(table), N, D, K, p(b) if b is not None else None,
+                                            p(a) if a is not None else None, K, p(out), K, None)
+    assert rc == expect_rc, rc
+    if rc:
+        return None
+    assert (out[N * K:] == np.float32(-777.0)).all()
+    return out[:N * K].reshape(N, K)
+
+
 def stream_probe(x, out_bytes, guard=32, expect_rc=0):
     """exact_stream_probe_f32 on a flat fp32 array -> the bytes it wrote."""
     x = f32(x).reshape(-1)

@@ -24,6 +24,8 @@ def test_pack_unpack(bits, N, G):
     x = (rng.standard_normal((N, G)) * 3).astype(F32)
     if N > 4:
         x[2] = 0.75                                          # a constant row
+        x[3] = 0.0
+        x[3, ::2] = 1e-45                                    # a spread whose reciprocal overflows: scale = inf
     u = rng.random((N, G), dtype=F32)
     want = o.quantize_activation(x, bits, u)
     packed, s32, m32, sbf, mbf = e.minmax_pack(x, bits, u)
@@ -342,3 +344,42 @@ def test_pack_geometry_candidates():
     assert extq.pack_geometry_candidates(2048) == []
     t = torch.zeros(4, 256)
     assert extq._pack_geometry(t, 2) == 0                      # host tensors (emulated runs) are never tuned
+
+
+@pytest.mark.parametrize("N,D,K", [(1, 4, 1), (33, 8, 5), (70, 256, 256), (40, 128, 40), (65, 100, 47), (31, 604, 332),
+                                   (64, 256, 300), (97, 48, 257), (130, 256, 41)])
+def test_tall_gemm(N, D, K):
+    """exact_tall_gemm_bf16_f32 = X . M (+ bias) (+ addend).  Small integers: every
+    bf16 piece, product and partial sum is exact, so the result must be the
+    integer product bit for bit -- a wrong fragment, column slab or tile offset
+    shows; random data of mixed magnitudes within fp32 accumulation error of
+    float64 (a dropped low-order piece would not be); M handed over transposed
+    and with a row stride; the output as its own addend."""
+    rng = np.random.default_rng(N + D + K)
+    X = rng.integers(-6, 7, (N, D)).astype(F32)
+    M = rng.integers(-6, 7, (D, K)).astype(F32)
+    bias = rng.integers(-9, 10, K).astype(F32)
+    add = rng.integers(-9, 10, (N, K)).astype(F32)
+    exact = X.astype(np.float64) @ M.astype(np.float64)
+    assert np.array_equal(e.tall_gemm(X, M), exact.astype(F32))
+    assert np.array_equal(e.tall_gemm(X, M, transposed=True, ld=D + 3), exact.astype(F32))
+    assert np.array_equal(e.tall_gemm(X, M, ld=K + 5), exact.astype(F32))
+    assert np.array_equal(e.tall_gemm(X, M, bias=bias), (exact + bias).astype(F32))
+    assert np.array_equal(e.tall_gemm(X, M, bias=bias, addend=add), (exact + bias + add).astype(F32))
+    assert np.array_equal(e.tall_gemm(X, M, addend=add, in_place=True), (exact + add).astype(F32))
+    X = (rng.standard_normal((N, D)) * np.exp(rng.uniform(-4, 4, (N, 1)))).astype(F32)
+    M = (rng.standard_normal((D, K)) * np.exp(rng.uniform(-4, 4, (1, K)))).astype(F32)
+    want = X.astype(np.float64) @ M.astype(np.float64)
+    bound = np.abs(X).astype(np.float64) @ np.abs(M).astype(np.float64)
+    assert (np.abs(e.tall_gemm(X, M) - want) <= 1e-6 * bound + 1e-30).all()
+
+
+def test_tall_gemm_limits():
+    X, M = np.zeros((8, 8), F32), np.zeros((8, 8), F32)
+    assert e.emu().exact_tall_gemm_table_nbytes(0, 8) == 0 and e.emu().exact_tall_gemm_table_nbytes(8, 5000) == 0
+    assert e.emu().exact_tall_gemm_table_nbytes(256, 256) == 16 * (1 + 16 * 8 * 3 * 64)
+    assert e.emu().exact_tall_gemm_bf16_f32(e.p(np.zeros((4, 6), F32)), e.p(np.zeros(1024, F32)), 4, 6, 8, None, None, 8,
+                                            e.p(np.zeros((4, 8), F32)), 8, None) == -3        # D % 4 != 0
+    assert e.emu().exact_tall_gemm_bf16_f32(e.p(X), e.p(np.zeros(4096, F32)), 8, 8, 8, None, None, 8, e.p(np.zeros((8, 8), F32)), 7,
+                                            None) == -3                                              # ldo < K
+    assert e.emu().exact_tall_gemm_bf16_f32(None, None, 0, 8, 8, None, None, 8, None, 8, None) == 0   # N == 0: nothing to do

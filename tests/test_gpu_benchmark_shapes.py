@@ -56,6 +56,78 @@ def test_weight_gradient_is_the_integer_product_at_benchmark_size(cuda, N, K, D,
     assert torch.equal(bf.weight_gradient(wide_dy[:, 2:2 + K], wide_x[:, 5:5 + D]), want)
 
 
+# (D, K) of the dense products x . M of the benchmark models: F.linear with M = W^T, the input gradient with M = W,
+# and the first SAGE layer's x [R | W_l^T]; plus widths that cut the 256-column slabs and the 32-column tiles unevenly
+GEMM_SHAPES = [(256, 256), (128, 256), (256, 40), (100, 256), (256, 47), (604, 332), (256, 300), (64, 1024), (1024, 64), (8, 8)]
+
+
+@pytest.mark.parametrize("N", BIG)
+@pytest.mark.parametrize("D,K", GEMM_SHAPES)
+def test_tall_gemm_is_the_integer_product_at_benchmark_size(cuda, N, D, K):
+    """exact_tall_gemm_bf16_f32 through the shim on small integers: every bf16
+    piece, product and partial sum is exact, so the result equals the float64
+    product bit for bit -- a wrong fragment, slab or tile offset, or a row missed,
+    shows.  With the matrix direct and transposed (a weight as F.linear holds
+    it), a bias, an addend and accumulation in place."""
+    if N * max(D, K) > 700_000_000:
+        pytest.skip("operands beyond what this test allocates")
+    print(f"case gemm N={N} D={D} K={K}", flush=True)
+    config.matrix_cores, config.tall_gemm_max_cols = "bf16", 4096
+    x = _ints((N, D), cuda, N + D, -5, 6)
+    m = _ints((D, K), cuda, D + K, -5, 6)
+    bias = _ints((K,), cuda, K, -9, 10)
+    want = (x.double() @ m.double())
+    got = bf.tall_matmul(x, m)
+    assert got.shape == (N, K) and torch.equal(got, want.float())
+    assert hasattr(m, "_exact_gemm_table")                      # the library kernel ran, not the framework's GEMM
+    weight = m.t().contiguous()                                 # [K, D]
+    assert torch.equal(bf.tall_matmul(x, weight, transposed=True, bias=bias), (want + bias.double()).float())
+    wide = torch.full((N, K + 6), float("nan"), device=cuda)
+    add = _ints((N, K), cuda, 5, -9, 10)
+    wide[:, 3:3 + K] = add
+    view = wide[:, 3:3 + K]
+    out = bf.tall_matmul(x, m, addend=view, into=view)          # accumulate into a strided view
+    assert out is view and torch.equal(view, (want + add.double()).float())
+    assert torch.isnan(wide[:, :3]).all() and torch.isnan(wide[:, 3 + K:]).all()
+
+
+@pytest.mark.parametrize("N,D,K", [(169343, 256, 256), (50000, 604, 332), (20000, 1024, 1024), (16384, 4096, 32), (16385, 32, 4096)])
+def test_tall_gemm_accuracy_and_the_framework_gemm(cuda, N, D, K):
+    """Random operands with rows and columns of very different size: within 1e-6
+    of the sum of the absolute terms of the float64 product (a dropped low-order
+    bf16 piece would miss that by far), and as close to it as the framework's
+    fp32 GEMM is."""
+    print(f"case gemm accuracy N={N} D={D} K={K}", flush=True)
+    config.matrix_cores, config.tall_gemm_max_cols = "bf16", 4096
+    g = torch.Generator(device=cuda).manual_seed(N + D)
+    x = torch.randn(N, D, generator=g, device=cuda) * torch.exp(8 * torch.rand(N, 1, generator=g, device=cuda) - 4)
+    m = torch.randn(D, K, generator=g, device=cuda) * torch.exp(8 * torch.rand(1, K, generator=g, device=cuda) - 4)
+    got = bf.tall_matmul(x, m)
+    assert hasattr(m, "_exact_gemm_table")
+    rows = torch.arange(0, N, max(1, N // 4096), device=cuda)
+    want = x[rows].double() @ m.double()
+    bound = x[rows].abs().double() @ m.abs().double()
+    mine = (got[rows].double() - want).abs()
+    assert (mine <= 1e-6 * bound + 1e-30).all()
+    theirs = (x[rows].mm(m).double() - want).abs()
+    assert (mine / (bound + 1e-30)).max().item() <= 4 * max((theirs / (bound + 1e-30)).max().item(), 2.0 ** -24)
+
+
+def test_tall_gemm_reprepares_a_changed_matrix(cuda):
+    """The fragment table is remembered on the matrix and rebuilt when it changes in place (an optimiser step)."""
+    config.matrix_cores = "bf16"
+    x = _ints((20000, 64), cuda, 1)
+    w = torch.nn.Parameter(_ints((48, 64), cuda, 2))
+    with torch.no_grad():
+        first = bf.tall_matmul(x, w, transposed=True)
+        assert torch.equal(first, x.mm(w.t()))
+        w.add_(1.0)
+        assert torch.equal(bf.tall_matmul(x, w, transposed=True), x.mm(w.t()))
+    config.matrix_cores = "fp32"
+    with torch.no_grad():
+        assert torch.equal(bf.tall_matmul(x, w, transposed=True), x.mm(w.t()))   # the framework's GEMM
+
+
 @pytest.mark.parametrize("cores", ["bf16", "fp32"])
 @pytest.mark.parametrize("N,K,D", [(20000, 1024, 1024), (16384, 1000, 513), (50000, 1, 1), (30011, 7, 1024), (169343, 256, 256)])
 def test_weight_gradient_limits_of_the_wrapper(cuda, N, K, D, cores):

@@ -41,6 +41,34 @@ def test_fused_pack_and_unpack_bit_exact(cuda, bits, N, G):
 
 
 @pytest.mark.parametrize("bits", [1, 2, 4, 8])
+@pytest.mark.parametrize("N,G", [(37, 25), (130, 256), (20, 602)])
+def test_constant_rows_and_rows_whose_scale_overflows(cuda, bits, N, G):
+    """Rows the quantiser's round-and-clamp sees as NaN (constant row: 0 * inf)
+    and as +inf (a spread so small that its reciprocal overflows; the conversion
+    saturates and the byte keeps the low bits of INT_MAX), next to ordinary
+    rows: one-launch and two-step forms, bit-exact against the oracle."""
+    x = host_randn((N, G), 5 + N) * F32(2.0)
+    x[1::5] = F32(0.75)
+    x[2::5] = 0.0
+    x[2::5, ::2] = F32(1e-45)
+    x[3::5] = F32(-3.0)
+    x[3::5, 1::3] = np.nextafter(F32(-3.0), F32(0.0))       # one ulp of spread: a finite, large scale
+    u = host_noise((N, G), 9 + N + bits)
+    want_packed, _, want_sbf, want_mbf, want_scale, want_min = o.quantize_activation(x, bits, u)
+    assert np.isinf(want_scale).sum() >= 2 * (N // 5)
+    config.noise_source = FixedNoise([torch.from_numpy(u), torch.from_numpy(u)])
+    packed, sbf, mbf, s32, m32 = extq.minmax_pack(dev(x), bits, want_fp32=True)
+    assert bytes_equal(s32, want_scale) and bytes_equal(m32, want_min)
+    assert bytes_equal(packed, want_packed)
+    tmn, tmx = extq.row_minmax(dev(x))
+    two_step = extq.pack_single_precision(dev(x), tmn, tmx, dev(want_scale), bits, True)
+    assert bytes_equal(two_step, want_packed)
+    got = extq.unpack_bf16param(packed, bits, sbf, mbf, N, G)
+    with np.errstate(all="ignore"):
+        assert bytes_equal(got, o.dequantize_activation(want_packed, bits, want_sbf, want_mbf, (N, G)))
+
+
+@pytest.mark.parametrize("bits", [1, 2, 4, 8])
 @pytest.mark.parametrize("N,G", [(37, 25), (777, 256), (61, 602), (9, 1500)])
 def test_two_step_pack_matches_reference_signature(cuda, bits, N, G):
     """ext_quantization.pack_single_precision(data, min, max, scale, bits, stochastic)."""

@@ -188,6 +188,22 @@ def test_spill_is_replicated_not_clamped():
     assert p4[0] == 0                                 # 16 << 4 leaves the byte
 
 
+def test_overflowing_scale_saturates_like_the_conversion():
+    """A row whose spread is so small that the reciprocal overflows: scale = inf,
+    the minimum gives 0 * inf = NaN -> code 0, every other element inf, which
+    __float2int_rn (cvt.rni.s32.f32, clamped to the int32 range) turns into
+    INT_MAX; the uint8 accumulator keeps the low byte of INT_MAX << (row * bits)."""
+    tiny = F32(1e-45)
+    x = np.array([[0, tiny, 0, tiny], [tiny, 0, tiny, tiny]], F32)
+    mn, mx = o.row_min_max(x)
+    for bits, want in ((8, [0, 0xFF, 0, 0xFF, 0xFF, 0, 0xFF, 0xFF]), (2, [0xFC, 0xFF, 0xFC, 0xFF]),
+                       (1, [0xFE, 0xFF, 0xFE, 0xFF]), (4, [0xF0, 0xFF, 0xF0, 0xFF])):
+        sc = o.compute_scale(mn, mx, bits)
+        assert np.isinf(sc).all()
+        p = _pack_both(x, mn, sc, bits, np.full(x.shape, 0.25, F32))
+        assert p[:-1].tolist() == want and p[-1] == 0
+
+
 def test_stochastic_rounding_is_unbiased():
     # E_u[q] = (x - mn) * scale: mean error < 1e-3 over 1e6 draws, supplied and Philox noise
     draws = 1_000_000
