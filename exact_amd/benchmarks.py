@@ -569,7 +569,7 @@ def _profile_target(argv=None):
                                       "rp_pack", "spmm", "copy", "probe", "dw"])
     ap.add_argument("--fp32-cores", action="store_true", help="dw only: the fp32 matrix-core kernel instead of the bf16 one")
     ap.add_argument("--cold", action="store_true",
-                    help="unpack only: every launch reads another copy of the packed stream (24 copies, none of it cached)")
+                    help="unpack only: every launch reads another copy of the packed stream (48 copies, 0.5 GB at 2 bits: none of it cached)")
     ap.add_argument("--rp-path", choices=["fp32", "split", "signs"], default="signs",
                     help="rp_* only: the fp32 matrix-core instruction on a Gaussian matrix, the bf16 instruction on split "
                          "operands (Gaussian matrix), or on the signs of a +-1/sqrt(k) matrix (the default path)")
@@ -616,7 +616,7 @@ def _profile_target(argv=None):
         rowptr, col, value = adj.csr()
         spmm_x = torch.randn((n_nodes, args.width or G), generator=gen, device=dev)
         spmm_reduce = "sum" if kind == "gcn" else "mean"
-    packs = [packed] + [packed.clone() for _ in range(23)] if args.cold else [packed]
+    packs = [packed] + [packed.clone() for _ in range(47)] if args.cold else [packed]
     dw_out = torch.empty((G, G), device=dev)
     dw_entry = L.exact_linear_dw_f32 if args.fp32_cores else L.exact_linear_dw_bf16_f32
     fns = {
