@@ -226,7 +226,7 @@ def kernel_extras(x, log):
         bias = torch.randn(G, device=x.device)
         flops = 2.0 * N * G * G
         gemm_bytes = 8 * N * G + 4 * G * G
-        config.tall_gemm_max_cols = 4096
+        config.tall_gemm_min_depth = 1
         w40 = torch.randn(40, G, device=x.device) / G ** 0.5
         for cores in ("bf16", "fp32"):
             config.matrix_cores = cores
@@ -529,10 +529,12 @@ def _epoch_main(argv):
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--epochs-only", action="store_true", help="leave out the separate SpMM timings after the epochs")
-    ap.add_argument("--set", action="append", default=[], metavar="FIELD=0|1",
-                    help="a boolean field of exact_amd.config to set for the run, e.g. --set sage_single_node=0")
+    ap.add_argument("--set", action="append", default=[], metavar="FIELD=VALUE",
+                    help="a boolean (0 | 1) or integer field of exact_amd.config to set for the run, e.g. "
+                         "--set sage_single_node=0 --set tall_gemm_min_rows=1000000000")
     args = ap.parse_args(argv)
-    overrides = {f: bool(int(v)) for f, v in (item.split("=", 1) for item in args.set)}
+    overrides = {f: (bool(int(v)) if isinstance(getattr(config, f), bool) else int(v))
+                 for f, v in (item.split("=", 1) for item in args.set)}
 
     def log(*a):
         print(*a, file=sys.stderr, flush=True)

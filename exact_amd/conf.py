@@ -99,9 +99,13 @@ _EXTRA_FIELDS = {
     # matrix-core kernel (config.matrix_cores == "bf16") from this many rows on;
     # shorter operands keep the framework's GEMM, which is as fast there.
     "tall_gemm_min_rows": 16384,
-    # ... and up to this many output columns: measured against the framework's
-    # fp32 GEMM the kernel is 20 - 25 % faster at 40 - 47 columns and equal at 256.
-    "tall_gemm_max_cols": 64,
+    # ... when the result has at most 64 columns (20 - 35 % faster than the
+    # framework's fp32 GEMM there) or the reduction runs over at least this many
+    # features (10 - 20 % faster at 256 and 604; slower at 100 - 128).
+    "tall_gemm_min_depth": 192,
+    # ... and, for such wide results, at most this many rows: at 2.4 M rows the
+    # framework's GEMM reaches 127 TFLOP/s and the two are equal.
+    "tall_gemm_max_rows_wide": 1000000,
 }
 
 

@@ -110,7 +110,9 @@ def tall_matmul(x, matrix, transposed=False, bias=None, addend=None, into=None):
     ([D, K]) or, with transposed=True, the transpose of `matrix` ([K, D]: a weight
     as F.linear holds it).  `into` names the result tensor; it may be `addend`
     itself (accumulate in place).  Tall fp32 device operands with a narrow result
-    (config.tall_gemm_min_rows, config.tall_gemm_max_cols) take the library's
+    (config.tall_gemm_min_rows; a result of at most 64 columns or a reduction over
+    at least config.tall_gemm_min_depth features of at most
+    config.tall_gemm_max_rows_wide rows) take the library's
     kernel (six bf16 matrix-core products per fp32 product, fp32 accuracy,
     reproducible; config.matrix_cores == "bf16"); everything else the
     framework's GEMM."""
@@ -118,7 +120,9 @@ def tall_matmul(x, matrix, transposed=False, bias=None, addend=None, into=None):
     usable = (config.matrix_cores == "bf16" and x.dim() == 2 and matrix.dim() == 2 and x.dtype == torch.float32
               and matrix.dtype == torch.float32 and _checks.on_device(x) and _checks.on_device(matrix)
               and x.shape[1] == M.shape[0] and x.shape[0] >= config.tall_gemm_min_rows and x.shape[1] % 4 == 0
-              and 0 < x.shape[1] <= 4096 and 0 < M.shape[1] <= min(4096, config.tall_gemm_max_cols) and x.is_contiguous() and x.data_ptr() % 16 == 0
+              and 0 < x.shape[1] <= 4096 and 0 < M.shape[1] <= 4096
+              and (M.shape[1] <= 64 or (x.shape[1] >= config.tall_gemm_min_depth and x.shape[0] <= config.tall_gemm_max_rows_wide))
+              and x.is_contiguous() and x.data_ptr() % 16 == 0
               and matrix.stride(1) == 1 and matrix.stride(0) >= matrix.shape[1]
               and (bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == M.shape[1]
                                     and _checks.on_device(bias)))

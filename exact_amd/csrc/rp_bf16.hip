@@ -341,24 +341,18 @@ __global__ __launch_bounds__(kWave) void rp_fwd_pack_bf16_kernel(const RpPackArg
 // out[N, K] = X[N, D] . M[D, K] (+ bias[K]) (+ addend[N, K]) for the linear maps of a
 // layer (F.linear and the input gradient of linear_backward, backward_func.cc:83-87):
 // the forward loop above with M split in three (six bf16 products per fp32
-// product, fp32 accuracy), up to eight column tiles per wavefront -- wider
-// matrices take one launch per slab of 256 columns -- and an epilogue that adds
+// product, fp32 accuracy), up to four column tiles per wavefront -- wider
+// matrices take one launch per slab of 128 columns -- and an epilogue that adds
 // a bias row and / or a matrix (which may be `out` itself: every element is read
 // and written by the same lane).  The fragments of M come from
 // exact_tall_gemm_prepare_bf16, which also takes M transposed (a weight as
 // F.linear holds it).  No atomics: the result does not depend on the launch.
-#ifndef EXACT_GEMM_SLAB_TILES
-#define EXACT_GEMM_SLAB_TILES 4
-#endif
-#ifndef EXACT_GEMM_ROW_TILES
-#define EXACT_GEMM_ROW_TILES 1
-#endif
-#ifndef EXACT_GEMM_STEPS
-#define EXACT_GEMM_STEPS 4
-#endif
-constexpr int kGemmSlabTiles = EXACT_GEMM_SLAB_TILES;  // column tiles (of 32) one launch covers, at most 8
-constexpr int kGemmRowTiles = EXACT_GEMM_ROW_TILES;    // row tiles (of 32) per wavefront
-constexpr int kGemmSteps = EXACT_GEMM_STEPS;           // k-steps whose loads are issued together
+constexpr int kGemmSlabTiles = 4;  // column tiles (of 32) one launch covers
+constexpr int kGemmRowTiles = 1;   // row tiles (of 32) per wavefront in the form without LDS
+constexpr int kGemmSteps = 4;      // k-steps whose loads are issued together there
+// Slabs that fill their launch share the fragments through LDS (tall_gemm_lds_bf16_kernel): results of up to two
+// column tiles as one slab with four k-steps per chunk, wider ones in slabs of four tiles with two steps per chunk
+// (measured: 64 against 77 us at 256 -> 40, 200 against 230 at 256 -> 256; the other splits tried were slower).
 
 __global__ __launch_bounds__(kBlock) void gemm_prepare_kernel(const float* __restrict__ M, int64_t ld, int transposed,
                                                               int D, int K, u32x4* __restrict__ table) {
@@ -462,6 +456,98 @@ __global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __re
           __builtin_nontemporal_store(val, out + n * ldo + col);
         }
       }
+  }
+}
+
+// The same product with the fragments of M shared by a workgroup: four wavefronts (128 rows) copy the fragments
+// of KS k-steps x NT column tiles into LDS once and all read them from there, so the L2 sees a quarter of the
+// fragment traffic and the wavefronts' fragment loads become LDS reads.  For results wider than a few tiles, where
+// every wavefront of the form above streams the whole slab of M through the vector memory pipeline.
+template <int NT, int KS>
+__global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float* __restrict__ X,
+                                                                    const u32x4* __restrict__ table, int64_t N, int D,
+                                                                    int K, int tiles, int tile0,
+                                                                    const float* __restrict__ bias, const float* addend,
+                                                                    int64_t ldc, float* out, int64_t ldo) {
+  HIP_DYNAMIC_SHARED(u32x4, shared_frags)  // [KS][NT][3][64]
+  constexpr int kUnits = KS * NT * 3 * kWave;             // 16-byte units per chunk
+  constexpr int kPerThread = kUnits / kBlock;             // KS * NT * 3 / 4
+  static_assert(kUnits % kBlock == 0, "whole units per thread");
+  constexpr int kStepUnits = NT * 3 * kWave;              // contiguous in the table for one k-step
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kTile;
+  const u32x4* frags = table + 1;
+  const int64_t my_row = (row0 + l32 < N) ? row0 + l32 : N - 1;
+  const float* xrow = X + my_row * D;
+  const int total = (D + kStepFeatures - 1) / kStepFeatures;
+  floatx16 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+
+  for (int s0 = 0; s0 < total; s0 += KS) {
+    float a[KS][8];
+    if ((s0 + KS) * kStepFeatures <= D) {  // wave-uniform: the KS steps lie inside the row, nothing to mask
+#pragma unroll
+      for (int sb = 0; sb < KS; ++sb) load8<4>(xrow, (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb]);
+    } else {
+#pragma unroll
+      for (int sb = 0; sb < KS; ++sb) load8<4>(xrow, (s0 + sb) * kStepFeatures + 8 * half, D, a[sb]);
+    }
+    // this thread's share of the chunk's fragments: global -> registers -> LDS
+    u32x4 mine[kPerThread];
+#pragma unroll
+    for (int u = 0; u < kPerThread; ++u) {
+      const int c = u * kBlock + static_cast<int>(threadIdx.x);  // unit of the chunk
+      const int sb = c / kStepUnits, within = c - sb * kStepUnits;
+      const int st = (s0 + sb < total) ? s0 + sb : s0;            // a step past the row meets zeros of X
+      mine[u] = frags[(static_cast<int64_t>(st) * tiles + tile0) * 3 * kWave + within];
+    }
+    __syncthreads();  // the previous chunk has been read by every wavefront
+#pragma unroll
+    for (int u = 0; u < kPerThread; ++u) shared_frags[u * kBlock + threadIdx.x] = mine[u];
+    __syncthreads();
+#pragma unroll
+    for (int sb = 0; sb < KS; ++sb) {
+      const Split8 pieces = split3x8(a[sb]);
+      u32x4 b[NT][3];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int p = 0; p < 3; ++p) b[nt][p] = shared_frags[((sb * NT + nt) * 3 + p) * kWave + lane];
+      // the six products of step_product<3>, in its order for every tile, issued tile after tile: consecutive
+      // matrix-core instructions write different accumulators and none waits for its predecessor
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.mid, b[nt][1], acc[nt]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.lo, b[nt][0], acc[nt]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.hi, b[nt][2], acc[nt]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.mid, b[nt][0], acc[nt]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.hi, b[nt][1], acc[nt]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.hi, b[nt][0], acc[nt]);
+    }
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int col = (tile0 + nt) * kTile + l32;
+    const float b = (bias != nullptr && col < K) ? bias[col] : 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int64_t n = row0 + 8 * (v / 4) + 4 * half + (v % 4);
+      if (n < N && col < K) {
+        float val = acc[nt][v];
+        if (bias != nullptr) val = val + b;
+        if (addend != nullptr) val = val + addend[n * ldc + col];
+        __builtin_nontemporal_store(val, out + n * ldo + col);
+      }
+    }
   }
 }
 
@@ -775,23 +861,33 @@ int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64
   const int tiles = (kk + kTile - 1) / kTile;
   const int64_t rows_per_wave = static_cast<int64_t>(kTile) * kGemmRowTiles;
   const dim3 grid(static_cast<unsigned>((N + rows_per_wave - 1) / rows_per_wave)), block(kWave);
+  const dim3 lgrid(static_cast<unsigned>((N + 4 * kTile - 1) / (4 * kTile))), lblock(kBlock);  // four wavefronts, 128 rows
+#define EXACT_GEMM_LDS(NTV, KSV)                                                                                    \
+  hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<NTV, KSV>), lgrid, lblock, sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, \
+                     tiles, tile0, bias, addend, ldc, out, ldo)
+#define EXACT_GEMM_GO(NTV)                                                                                          \
+  hipLaunchKernelGGL((tall_gemm_bf16_kernel<kGemmRowTiles, NTV, kGemmSteps>), grid, block, 0, s, X, t, N, \
+                     d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
+  if (tiles == 2) {
+    const int tile0 = 0;
+    EXACT_GEMM_LDS(2, 4);
+    return launch_status();
+  }
   for (int tile0 = 0; tile0 < tiles; tile0 += kGemmSlabTiles) {
     const int nt = tiles - tile0 < kGemmSlabTiles ? tiles - tile0 : kGemmSlabTiles;
-#define EXACT_GEMM_GO(NTV)                                                                                          \
-  hipLaunchKernelGGL((tall_gemm_bf16_kernel<kGemmRowTiles, (NTV <= kGemmSlabTiles ? NTV : 1), kGemmSteps>), grid, block, 0, s, X, t, N, \
-                     d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
+    if (nt == 4) {
+      EXACT_GEMM_LDS(4, 2);
+      continue;
+    }
     switch (nt) {
       case 1: EXACT_GEMM_GO(1); break;
       case 2: EXACT_GEMM_GO(2); break;
       case 3: EXACT_GEMM_GO(3); break;
-      case 4: EXACT_GEMM_GO(4); break;
-      case 5: EXACT_GEMM_GO(5); break;
-      case 6: EXACT_GEMM_GO(6); break;
-      case 7: EXACT_GEMM_GO(7); break;
-      default: EXACT_GEMM_GO(8); break;
+      default: EXACT_GEMM_GO(4); break;
     }
-#undef EXACT_GEMM_GO
   }
+#undef EXACT_GEMM_LDS
+#undef EXACT_GEMM_GO
   return launch_status();
 }
 

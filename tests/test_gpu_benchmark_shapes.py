@@ -72,7 +72,7 @@ def test_tall_gemm_is_the_integer_product_at_benchmark_size(cuda, N, D, K):
     if N * max(D, K) > 700_000_000:
         pytest.skip("operands beyond what this test allocates")
     print(f"case gemm N={N} D={D} K={K}", flush=True)
-    config.matrix_cores, config.tall_gemm_max_cols = "bf16", 4096
+    config.matrix_cores, config.tall_gemm_min_depth, config.tall_gemm_max_rows_wide = "bf16", 1, 10 ** 9
     x = _ints((N, D), cuda, N + D, -5, 6)
     m = _ints((D, K), cuda, D + K, -5, 6)
     bias = _ints((K,), cuda, K, -9, 10)
@@ -98,7 +98,7 @@ def test_tall_gemm_accuracy_and_the_framework_gemm(cuda, N, D, K):
     bf16 piece would miss that by far), and as close to it as the framework's
     fp32 GEMM is."""
     print(f"case gemm accuracy N={N} D={D} K={K}", flush=True)
-    config.matrix_cores, config.tall_gemm_max_cols = "bf16", 4096
+    config.matrix_cores, config.tall_gemm_min_depth, config.tall_gemm_max_rows_wide = "bf16", 1, 10 ** 9
     g = torch.Generator(device=cuda).manual_seed(N + D)
     x = torch.randn(N, D, generator=g, device=cuda) * torch.exp(8 * torch.rand(N, 1, generator=g, device=cuda) - 4)
     m = torch.randn(D, K, generator=g, device=cuda) * torch.exp(8 * torch.rand(1, K, generator=g, device=cuda) - 4)

@@ -404,9 +404,9 @@ SAGE_FORMS = {
     "node+backward": dict(sage_single_node=True, sage_reassociate_backward=True, sage_aggregate_projected=False),
     "node+both": dict(sage_single_node=True, sage_reassociate_backward=True, sage_aggregate_projected=True),
     # every dense product of the layer through the library's bf16 matrix-core GEMM (rows of any count qualify)
-    "chain, library GEMMs": dict(sage_single_node=False, tall_gemm_min_rows=1, tall_gemm_max_cols=4096),
+    "chain, library GEMMs": dict(sage_single_node=False, tall_gemm_min_rows=1, tall_gemm_min_depth=1),
     "node+both, library GEMMs": dict(sage_single_node=True, sage_reassociate_backward=True, sage_aggregate_projected=True,
-                                     tall_gemm_min_rows=1, tall_gemm_max_cols=4096),
+                                     tall_gemm_min_rows=1, tall_gemm_min_depth=1),
 }
 
 
@@ -504,8 +504,8 @@ GCN_FORMS = {
     "chain": dict(gcn_single_node=False),
     "node": dict(gcn_single_node=True, gcn_aggregate_narrow=False),
     "node+narrow": dict(gcn_single_node=True, gcn_aggregate_narrow=True),
-    "chain, library GEMMs": dict(gcn_single_node=False, tall_gemm_min_rows=1, tall_gemm_max_cols=4096),
-    "node+narrow, library GEMMs": dict(gcn_single_node=True, gcn_aggregate_narrow=True, tall_gemm_min_rows=1, tall_gemm_max_cols=4096),
+    "chain, library GEMMs": dict(gcn_single_node=False, tall_gemm_min_rows=1, tall_gemm_min_depth=1),
+    "node+narrow, library GEMMs": dict(gcn_single_node=True, gcn_aggregate_narrow=True, tall_gemm_min_rows=1, tall_gemm_min_depth=1),
 }
 
 
