@@ -179,6 +179,11 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   constexpr float B = static_cast<float>((1 << BITS) - 1);
   __shared__ uint2 stage[WPT > 1 ? OPT * kBlock : 1];
   __shared__ f32x4 ybuf[ACT ? OPT * kBlock * 2 : 1];  // ACT: the activation output on its way to memory
+  // ACT with a normalisation ahead: mean, mult and shift of the G columns (dynamic LDS, 3 G floats, asked for by
+  // that launch only).  Every row needs them, so the workgroup fetches them once; read from memory per oct they
+  // cost three times the load instructions of x itself
+  HIP_DYNAMIC_SHARED(f32x4, norm_quads)  // declared in 16-byte units: the parameters are read as quads
+  float* norm_lds = reinterpret_cast<float*>(norm_quads);
 
   const int t = threadIdx.x;
   const int lpr = 1 << a.lpr_log2;
@@ -207,6 +212,17 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
   };
   // rows past the end re-read the last row and drop it
   const off_t row_ld_off = static_cast<off_t>(row_ok ? row_local : rows_here - 1) * G + static_cast<off_t>(8 * oct_base);
+
+  if constexpr (ACT) {
+    if (a.norm_mean != nullptr) {  // same for every lane of the launch: every wavefront reaches the barrier
+      for (int c = t; c < a.G; c += kBlock) {
+        norm_lds[c] = a.norm_mean[c];
+        norm_lds[a.G + c] = a.norm_mult[c];
+        norm_lds[2 * a.G + c] = a.norm_shift[c];
+      }
+      __syncthreads();
+    }
+  }
 
   float v[OPT][8];
   int nv[OPT];
@@ -256,9 +272,9 @@ __global__ __launch_bounds__(kBlock) void pack_kernel(const PackArgs a) {
           // training-mode batch norm of the column, statistics given:
           // weight * (x - mean) * invstd + bias with mult = weight * invstd
           float cm[8], cs[8], cb[8];
-          load_cached8(a.norm_mean + d0, cm);
-          load_cached8(a.norm_mult + d0, cs);
-          load_cached8(a.norm_shift + d0, cb);
+          load_cached8(norm_lds + d0, cm);
+          load_cached8(norm_lds + a.G + d0, cs);
+          load_cached8(norm_lds + 2 * a.G + d0, cb);
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             float c = v[k][i] - cm[i];
@@ -645,10 +661,11 @@ static int pack_common(const float* x, const float* mn, const float* scale, cons
 // ---- ReLU + dropout + statistics + pack (ACT form) ---------------------------
 template <int BITS, int OPT, bool NOISE_IN>
 static void launch_act_variant(const PackArgs& a, bool full, dim3 grid, hipStream_t s) {
+  const size_t norm_bytes = a.norm_mean != nullptr ? sizeof(float) * 3 * static_cast<size_t>(a.G) : 0;  // G <= 1024: 12 KB
   if (full)
-    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, true, NOISE_IN, true, true>), grid, dim3(kBlock), 0, s, a);
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, true, NOISE_IN, true, true>), grid, dim3(kBlock), norm_bytes, s, a);
   else
-    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, false, NOISE_IN, true, true>), grid, dim3(kBlock), 0, s, a);
+    hipLaunchKernelGGL((pack_kernel<BITS, OPT, 4, false, NOISE_IN, true, true>), grid, dim3(kBlock), norm_bytes, s, a);
 }
 
 template <int BITS, bool NOISE_IN>
