@@ -550,7 +550,7 @@ def _profile_target(argv=None):
     `--pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs:
 
         python -m exact_amd.benchmarks pack --bits 2 --reps 100
-        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy,probe,dw} ...
+        python -m exact_amd.benchmarks {unpack,relu,dropout,relu_dropout_pack,bn_relu_dropout_pack,rp_fwd,rp_bwd,rp_pack,spmm,copy,probe,dw,gemm} ...
         python -m exact_amd.benchmarks epoch --config cfg3_gcn_int2 --epochs 5
 
     `copy` is a plain device-to-device copy of the same [rows, cols] fp32 tensor
@@ -568,7 +568,7 @@ def _profile_target(argv=None):
         return _epoch_main(argv[1:])
     ap = argparse.ArgumentParser(prog="python -m exact_amd.benchmarks")
     ap.add_argument("kernel", choices=["pack", "unpack", "relu", "dropout", "relu_dropout_pack", "bn_relu_dropout_pack", "rp_fwd", "rp_bwd",
-                                      "rp_pack", "spmm", "copy", "probe", "dw"])
+                                      "rp_pack", "spmm", "copy", "probe", "dw", "gemm"])
     ap.add_argument("--fp32-cores", action="store_true", help="dw only: the fp32 matrix-core kernel instead of the bf16 one")
     ap.add_argument("--cold", action="store_true",
                     help="unpack only: every launch reads another copy of the packed stream (48 copies, 0.5 GB at 2 bits: none of it cached)")
@@ -582,7 +582,7 @@ def _profile_target(argv=None):
     ap.add_argument("--supplied-noise", action="store_true")
     ap.add_argument("--config", choices=sorted(EPOCH_CONFIGS), default="cfg3_gcn_int2",
                     help="spmm only: the graph of this model configuration")
-    ap.add_argument("--width", type=int, default=0, help="spmm only: columns of the dense operand (0 = --cols)")
+    ap.add_argument("--width", type=int, default=0, help="spmm: columns of the dense operand; gemm: columns of the result (0 = --cols)")
     args = ap.parse_args(argv)
     dev = bench_device()
     L = _lib.lib()
@@ -621,7 +621,10 @@ def _profile_target(argv=None):
     packs = [packed] + [packed.clone() for _ in range(47)] if args.cold else [packed]
     dw_out = torch.empty((G, G), device=dev)
     dw_entry = L.exact_linear_dw_f32 if args.fp32_cores else L.exact_linear_dw_bf16_f32
+    gemm_w = torch.randn((args.width or G, G), generator=gen, device=dev) / G ** 0.5   # a weight [out, in]
     fns = {
+        # x W^T as a layer computes it: the library's bf16 matrix-core kernel where the shim selects it
+        "gemm": lambda i: ext_backward_func.tall_matmul(xs[i % 3], gemm_w, transposed=True),
         "dw": lambda i: dw_entry(xs[i % 3].data_ptr(), G, xs[(i + 1) % 3].data_ptr(), G, N, G, G, dw_out.data_ptr(), sp),
         "pack": lambda i: L.exact_minmax_pack_f32(xs[i % 3].data_ptr(), noise.data_ptr() if noise is not None else None, 1,
                                                   i, N, G, b, packed.data_ptr(), None, None, sbf.data_ptr(),

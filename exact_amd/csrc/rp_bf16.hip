@@ -463,7 +463,7 @@ __global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __re
 // of KS k-steps x NT column tiles into LDS once and all read them from there, so the L2 sees a quarter of the
 // fragment traffic and the wavefronts' fragment loads become LDS reads.  For results wider than a few tiles, where
 // every wavefront of the form above streams the whole slab of M through the vector memory pipeline.
-template <int NT, int KS>
+template <int RT, int NT, int KS>
 __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float* __restrict__ X,
                                                                     const u32x4* __restrict__ table, int64_t N, int D,
                                                                     int K, int tiles, int tile0,
@@ -477,25 +477,38 @@ __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float*
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const int half = lane >> 5, l32 = lane & 31;
-  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * kTile;
+  // a wavefront owns RT row tiles, so that a fragment read from LDS could serve RT products.  Measured at
+  // [169343, 256] x [256, 256]: 201 us with one row tile, 287 with two, 280 with three -- the kernel lives on
+  // the number of wavefronts in flight (registers per wavefront), not on fragment reads; RT = 1 is what is launched
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * (kTile * RT);
   const u32x4* frags = table + 1;
-  const int64_t my_row = (row0 + l32 < N) ? row0 + l32 : N - 1;
-  const float* xrow = X + my_row * D;
+  const float* xrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int64_t r = row0 + rt * kTile + l32;
+    xrow[rt] = X + (r < N ? r : N - 1) * D;
+  }
   const int total = (D + kStepFeatures - 1) / kStepFeatures;
-  floatx16 acc[NT];
+  floatx16 acc[RT][NT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[nt][v] = 0.f;
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[rt][nt][v] = 0.f;
 
   for (int s0 = 0; s0 < total; s0 += KS) {
-    float a[KS][8];
+    float a[KS][RT][8];
     if ((s0 + KS) * kStepFeatures <= D) {  // wave-uniform: the KS steps lie inside the row, nothing to mask
 #pragma unroll
-      for (int sb = 0; sb < KS; ++sb) load8<4>(xrow, (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb]);
+      for (int sb = 0; sb < KS; ++sb)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb][rt]);
     } else {
 #pragma unroll
-      for (int sb = 0; sb < KS; ++sb) load8<4>(xrow, (s0 + sb) * kStepFeatures + 8 * half, D, a[sb]);
+      for (int sb = 0; sb < KS; ++sb)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, D, a[sb][rt]);
     }
     // this thread's share of the chunk's fragments: global -> registers -> LDS
     u32x4 mine[kPerThread];
@@ -512,26 +525,29 @@ __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float*
     __syncthreads();
 #pragma unroll
     for (int sb = 0; sb < KS; ++sb) {
-      const Split8 pieces = split3x8(a[sb]);
       u32x4 b[NT][3];
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int p = 0; p < 3; ++p) b[nt][p] = shared_frags[((sb * NT + nt) * 3 + p) * kWave + lane];
-      // the six products of step_product<3>, in its order for every tile, issued tile after tile: consecutive
-      // matrix-core instructions write different accumulators and none waits for its predecessor
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.mid, b[nt][1], acc[nt]);
+      for (int rt = 0; rt < RT; ++rt) {
+        const Split8 pieces = split3x8(a[sb][rt]);
+        // the six products of step_product<3>, in its order for every tile, issued tile after tile: consecutive
+        // matrix-core instructions write different accumulators and none waits for its predecessor
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.lo, b[nt][0], acc[nt]);
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = mfma_bf16(pieces.mid, b[nt][1], acc[rt][nt]);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.hi, b[nt][2], acc[nt]);
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = mfma_bf16(pieces.lo, b[nt][0], acc[rt][nt]);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.mid, b[nt][0], acc[nt]);
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = mfma_bf16(pieces.hi, b[nt][2], acc[rt][nt]);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.hi, b[nt][1], acc[nt]);
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = mfma_bf16(pieces.mid, b[nt][0], acc[rt][nt]);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma_bf16(pieces.hi, b[nt][0], acc[nt]);
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = mfma_bf16(pieces.hi, b[nt][1], acc[rt][nt]);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = mfma_bf16(pieces.hi, b[nt][0], acc[rt][nt]);
+      }
     }
   }
 #pragma unroll
@@ -539,15 +555,17 @@ __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float*
     const int col = (tile0 + nt) * kTile + l32;
     const float b = (bias != nullptr && col < K) ? bias[col] : 0.f;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int64_t n = row0 + 8 * (v / 4) + 4 * half + (v % 4);
-      if (n < N && col < K) {
-        float val = acc[nt][v];
-        if (bias != nullptr) val = val + b;
-        if (addend != nullptr) val = val + addend[n * ldc + col];
-        __builtin_nontemporal_store(val, out + n * ldo + col);
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t n = row0 + rt * kTile + 8 * (v / 4) + 4 * half + (v % 4);
+        if (n < N && col < K) {
+          float val = acc[rt][nt][v];
+          if (bias != nullptr) val = val + b;
+          if (addend != nullptr) val = val + addend[n * ldc + col];
+          __builtin_nontemporal_store(val, out + n * ldo + col);
+        }
       }
-    }
   }
 }
 
@@ -861,10 +879,15 @@ int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64
   const int tiles = (kk + kTile - 1) / kTile;
   const int64_t rows_per_wave = static_cast<int64_t>(kTile) * kGemmRowTiles;
   const dim3 grid(static_cast<unsigned>((N + rows_per_wave - 1) / rows_per_wave)), block(kWave);
-  const dim3 lgrid(static_cast<unsigned>((N + 4 * kTile - 1) / (4 * kTile))), lblock(kBlock);  // four wavefronts, 128 rows
+#ifndef EXACT_GEMM_LDS_ROW_TILES
+#define EXACT_GEMM_LDS_ROW_TILES 1
+#endif
+  constexpr int kLdsRowTiles = EXACT_GEMM_LDS_ROW_TILES;  // row tiles per wavefront in the LDS form
+  const int64_t lrows = static_cast<int64_t>(4) * kTile * kLdsRowTiles;  // four wavefronts
+  const dim3 lgrid(static_cast<unsigned>((N + lrows - 1) / lrows)), lblock(kBlock);
 #define EXACT_GEMM_LDS(NTV, KSV)                                                                                    \
-  hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<NTV, KSV>), lgrid, lblock, sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, \
-                     tiles, tile0, bias, addend, ldc, out, ldo)
+  hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<kLdsRowTiles, NTV, KSV>), lgrid, lblock, sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, \
+                     d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
 #define EXACT_GEMM_GO(NTV)                                                                                          \
   hipLaunchKernelGGL((tall_gemm_bf16_kernel<kGemmRowTiles, NTV, kGemmSteps>), grid, block, 0, s, X, t, N, \
                      d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
