@@ -46,7 +46,9 @@ def quantize_activation(x, bits, noise):
         t = (t + np.asarray(noise, F32)).astype(F32)
         t = (t - F32(0.5)).astype(F32)
         t = np.fmax(t, F32(0.0))
-        q = np.where(t >= F32(2147483648.0), 2147483647, np.rint(np.where(np.isinf(t), F32(0.0), t))).astype(np.int64)   # cvt.rni.s32.f32 saturates
+        # cvt.rni.s32.f32 clamps to the int32 range: +inf (a scale that overflowed fp16) gives INT_MAX
+        big = t >= F32(2147483648.0)
+        q = np.where(big, np.int64(2147483647), np.rint(np.where(big, F32(0.0), t)).astype(np.int64))
     N, G = x.shape
     wpt = 8 // bits
     n_round = N + (wpt - N % wpt) % wpt

@@ -99,16 +99,28 @@ def other_case(rng, n):
                 assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * max(1, np.abs(want).max())), ("sddmm", M, N, K)
     elif k == 2:    # rp
         N, D = int(rng.integers(1, 300)), int(rng.choice([7, 50, 100, 128, 256, 602])); kk = int(rng.integers(1, min(D, 128) + 1))
-        X = rng.standard_normal((N, D)).astype(F32); R = (rng.standard_normal((D, kk)) / np.sqrt(kk)).astype(F32)
-        a = e.rp_fwd(X, R); w = o.input2rp(X, R)
-        assert np.allclose(a, w, rtol=2e-5, atol=2e-5 * np.abs(w).max()), ("rp_fwd", N, D, kk)
-        b = e.rp_bwd(w, R); wb = o.rp2input(w, R)
-        assert np.allclose(b, wb, rtol=2e-5, atol=2e-5 * np.abs(wb).max()), ("rp_bwd", N, D, kk)
+        # the fp32 matrix-core instruction, or the bf16 one on split operands (any matrix) or on the signs of a +-c matrix
+        mode = str(rng.choice(["fp32", "bf16_split", "bf16_signs"]))
+        X = rng.standard_normal((N, D)).astype(F32)
+        if mode == "bf16_signs":
+            R = ((2.0 * rng.integers(0, 2, (D, kk)) - 1) / np.sqrt(kk)).astype(F32)
+        else:
+            R = (rng.standard_normal((D, kk)) / np.sqrt(kk)).astype(F32)
+        a = e.rp_fwd(X, R, mode=mode); w = o.input2rp(X, R)
+        assert np.allclose(a, w, rtol=2e-5, atol=2e-5 * np.abs(w).max()), ("rp_fwd", N, D, kk, mode)
+        b = e.rp_bwd(w, R, mode=mode); wb = o.rp2input(w, R)
+        assert np.allclose(b, wb, rtol=2e-5, atol=2e-5 * np.abs(wb).max()), ("rp_bwd", N, D, kk, mode)
+        if rng.integers(0, 4) == 0:     # the tall GEMM on the same operands (D a multiple of 4), with bias and addend
+            D4 = max(4, D // 4 * 4); Kg = int(rng.choice([1, 31, 40, 64, 100, 130, 256, 300]))
+            Xg = rng.integers(-6, 7, (N, D4)).astype(F32); Mg = rng.integers(-6, 7, (D4, Kg)).astype(F32)
+            bias = rng.integers(-9, 10, Kg).astype(F32); add = rng.integers(-9, 10, (N, Kg)).astype(F32)
+            want = (Xg.astype(np.float64) @ Mg.astype(np.float64) + bias + add).astype(F32)
+            assert np.array_equal(e.tall_gemm(Xg, Mg, bias=bias, addend=add, transposed=bool(rng.integers(0, 2))), want), ("gemm", N, D4, Kg)
         # projection + quantisation in one launch == the oracle's quantiser on the kernel's own product
         bits = int(rng.choice([1, 2, 4, 8])); supplied = bool(rng.integers(0, 2))
         seed, off = int(rng.integers(0, 2**63)), int(rng.integers(0, 2**40))
         noise = rng.random((N, kk), dtype=F32) if supplied else o.philox_noise_rows(seed, off, N, kk)
-        got = e.rp_minmax_pack(X, R, bits, noise if supplied else None, seed, off)
+        got = e.rp_minmax_pack(X, R, bits, noise if supplied else None, seed, off, mode=mode)
         wq = o.quantize_activation(a, bits, noise)
         assert np.array_equal(got[0][:-1], wq[0][:got[0].size - 1]) and np.array_equal(got[3], wq[2]) and np.array_equal(got[4], wq[3]), ("rp_pack", N, D, kk, bits, supplied)
     else:           # two-step pack with given min / scale, row_minmax

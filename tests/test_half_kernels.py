@@ -24,6 +24,7 @@ def test_pack_and_unpack_f16(N, G, bits, supplied):
     x = (rng.standard_normal((N, G)) * 3).astype(F16)
     if N > 2:
         x[1] = x[1, 0]                                   # constant row
+        x[2] = (rng.standard_normal(G) * 2e-6).astype(F16)   # a spread whose reciprocal overflows fp16: scale = inf (G > 1)
     noise = rng.random((N, G), dtype=F32) if supplied else o.philox_noise_rows(0xFEED, (2 << 32) + 8, N, G)
     packed, sc, mn = e.minmax_pack_f16(x, bits, noise if supplied else None, 0xFEED, (2 << 32) + 8)
     wp, ws, wm = oh.quantize_activation(x, bits, noise)

@@ -70,6 +70,18 @@ def test_unpack_matches_torch_half_arithmetic(bits):
     assert (err[ok] <= (step[ok, None] * 1.0 + np.abs(xn[ok].astype(F32)) * 2e-3 + 1e-3)).all()
 
 
+def test_overflowing_half_scale_saturates_like_the_conversion():
+    """A row whose spread is so small that its reciprocal overflows fp16: the scale is inf, the minimum
+    gives 0 * inf = NaN -> code 0, every other element +inf, which __float2int_rn
+    (cvt.rni.s32.f32, clamped to the int32 range) turns into INT_MAX; the uint8
+    accumulator keeps its low bits shifted by the row's position in the byte."""
+    x = np.array([[0.0, 5e-6, 0.0, 1e-5], [1.5e-5, 5e-6, 1.5e-5, 1e-5]], np.float16)      # spreads of 1e-5: 1 / spread > 65504
+    for bits, want in ((8, [0, 0xFF, 0, 0xFF, 0xFF, 0, 0xFF, 0xFF]), (2, [0xFC, 0xFF, 0xFC, 0xFF]), (1, [0xFE, 0xFF, 0xFE, 0xFF])):
+        packed, scale, mn = oh.quantize_activation(x, bits, np.full(x.shape, 0.25, np.float32))
+        assert np.isinf(scale.astype(np.float32)).all()
+        assert packed[:-1].tolist() == want and packed[-1] == 0
+
+
 def test_mask_ops_match_torch_half():
     rng = np.random.default_rng(5)
     x = (rng.standard_normal(1000) * 4).astype(F16)
