@@ -119,10 +119,10 @@ def tall_matmul(x, matrix, transposed=False, bias=None, addend=None, into=None):
     M = matrix.t() if transposed else matrix
     usable = (config.matrix_cores == "bf16" and x.dim() == 2 and matrix.dim() == 2 and x.dtype == torch.float32
               and matrix.dtype == torch.float32 and _checks.on_device(x) and _checks.on_device(matrix)
-              and x.shape[1] == M.shape[0] and x.shape[0] >= config.tall_gemm_min_rows and x.shape[1] % 4 == 0
+              and x.shape[1] == M.shape[0] and x.shape[0] >= config.tall_gemm_min_rows and x.shape[1] % 2 == 0
               and 0 < x.shape[1] <= 4096 and 0 < M.shape[1] <= 4096
               and (M.shape[1] <= 64 or (x.shape[1] >= config.tall_gemm_min_depth and x.shape[0] <= config.tall_gemm_max_rows_wide))
-              and x.is_contiguous() and x.data_ptr() % 16 == 0
+              and x.is_contiguous() and x.data_ptr() % 8 == 0
               and matrix.stride(1) == 1 and matrix.stride(0) >= matrix.shape[1]
               and (bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == M.shape[1]
                                     and _checks.on_device(bias)))

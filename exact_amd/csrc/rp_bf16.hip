@@ -385,7 +385,7 @@ __global__ __launch_bounds__(kBlock) void gemm_prepare_kernel(const float* __res
 // is the fastest split (two or three row tiles per wavefront -- every fragment of M then serves several
 // products -- cost more in occupancy than they save in fragment loads: 330 against 236 us at 256 x 256).  The
 // kernel then equals the framework's fp32 GEMM at 256 output columns and beats it by 20 - 25 % at 40 - 47.
-template <int RT, int NT, int KS>
+template <int VEC, int RT, int NT, int KS>
 __global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __restrict__ X,
                                                                const u32x4* __restrict__ table, int64_t N, int D, int K,
                                                                int tiles, int tile0, const float* __restrict__ bias,
@@ -416,12 +416,12 @@ __global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __re
 #pragma unroll
       for (int sb = 0; sb < KS; ++sb)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb][rt]);
+        for (int rt = 0; rt < RT; ++rt) load8<VEC>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb][rt]);
     } else {
 #pragma unroll
       for (int sb = 0; sb < KS; ++sb)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, D, a[sb][rt]);
+        for (int rt = 0; rt < RT; ++rt) load8<VEC>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, D, a[sb][rt]);
     }
 #pragma unroll
     for (int sb = 0; sb < KS; ++sb) {
@@ -463,7 +463,7 @@ __global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __re
 // of KS k-steps x NT column tiles into LDS once and all read them from there, so the L2 sees a quarter of the
 // fragment traffic and the wavefronts' fragment loads become LDS reads.  For results wider than a few tiles, where
 // every wavefront of the form above streams the whole slab of M through the vector memory pipeline.
-template <int RT, int NT, int KS>
+template <int VEC, int RT, int NT, int KS>
 __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float* __restrict__ X,
                                                                     const u32x4* __restrict__ table, int64_t N, int D,
                                                                     int K, int tiles, int tile0,
@@ -503,12 +503,12 @@ __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float*
 #pragma unroll
       for (int sb = 0; sb < KS; ++sb)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb][rt]);
+        for (int rt = 0; rt < RT; ++rt) load8<VEC>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, 0x7FFFFFFF, a[sb][rt]);
     } else {
 #pragma unroll
       for (int sb = 0; sb < KS; ++sb)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) load8<4>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, D, a[sb][rt]);
+        for (int rt = 0; rt < RT; ++rt) load8<VEC>(xrow[rt], (s0 + sb) * kStepFeatures + 8 * half, D, a[sb][rt]);
     }
     // this thread's share of the chunk's fragments: global -> registers -> LDS
     u32x4 mine[kPerThread];
@@ -868,11 +868,12 @@ int exact_tall_gemm_prepare_bf16(const float* M, int64_t ld, int transposed, int
 
 int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64_t D, int64_t K, const float* bias,
                              const float* addend, int64_t ldc, float* out, int64_t ldo, void* stream) {
-  if (N < 0 || D <= 0 || K <= 0 || D > 4096 || K > 4096 || D % 4 != 0) return EXACT_E_SHAPE;
+  if (N < 0 || D <= 0 || K <= 0 || D > 4096 || K > 4096 || D % 2 != 0) return EXACT_E_SHAPE;
   if (ldo < K || (addend && ldc < K)) return EXACT_E_SHAPE;
   if (N == 0) return EXACT_OK;
   if (!X || !table || !out) return EXACT_E_NULL;
-  if (!al16(table) || !al16(X)) return EXACT_E_ALIGN;
+  if (!al16(table) || !al8(X)) return EXACT_E_ALIGN;
+  const bool quads = D % 4 == 0 && al16(X);  // 16-byte loads of X, else 8-byte ones
   hipStream_t s = static_cast<hipStream_t>(stream);
   const u32x4* t = static_cast<const u32x4*>(table);
   const int d = static_cast<int>(D), kk = static_cast<int>(K);
@@ -886,11 +887,23 @@ int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64
   const int64_t lrows = static_cast<int64_t>(4) * kTile * kLdsRowTiles;  // four wavefronts
   const dim3 lgrid(static_cast<unsigned>((N + lrows - 1) / lrows)), lblock(kBlock);
 #define EXACT_GEMM_LDS(NTV, KSV)                                                                                    \
-  hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<kLdsRowTiles, NTV, KSV>), lgrid, lblock, sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, \
-                     d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
+  do {                                                                                                              \
+    if (quads)                                                                                                      \
+      hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<4, kLdsRowTiles, NTV, KSV>), lgrid, lblock,                     \
+                         sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, tiles, tile0, bias, addend, ldc, out, ldo); \
+    else                                                                                                            \
+      hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<2, kLdsRowTiles, NTV, KSV>), lgrid, lblock,                     \
+                         sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, tiles, tile0, bias, addend, ldc, out, ldo); \
+  } while (0)
 #define EXACT_GEMM_GO(NTV)                                                                                          \
-  hipLaunchKernelGGL((tall_gemm_bf16_kernel<kGemmRowTiles, NTV, kGemmSteps>), grid, block, 0, s, X, t, N, \
-                     d, kk, tiles, tile0, bias, addend, ldc, out, ldo)
+  do {                                                                                                              \
+    if (quads)                                                                                                      \
+      hipLaunchKernelGGL((tall_gemm_bf16_kernel<4, kGemmRowTiles, NTV, kGemmSteps>), grid, block, 0, s, X, t, N, d, kk, tiles, \
+                         tile0, bias, addend, ldc, out, ldo);                                                      \
+    else                                                                                                            \
+      hipLaunchKernelGGL((tall_gemm_bf16_kernel<2, kGemmRowTiles, NTV, kGemmSteps>), grid, block, 0, s, X, t, N, d, kk, tiles, \
+                         tile0, bias, addend, ldc, out, ldo);                                                      \
+  } while (0)
   if (tiles == 2) {
     const int tile0 = 0;
     EXACT_GEMM_LDS(2, 4);

@@ -377,7 +377,8 @@ int exact_rp_minmax_pack_bf16_f32(const float *X, const void *table, int mode, c
  * caller, valid while M is unchanged); M has row stride `ld` elements and is
  * read as M[d * ld + c], or as M[c * ld + d] when `transposed` is 1 (a weight
  * [K, D] as F.linear holds it).
- * exact_tall_gemm_bf16_f32: X contiguous [N, D], 16-byte aligned, D % 4 == 0,
+ * exact_tall_gemm_bf16_f32: X contiguous [N, D], D even, 8-byte aligned (16-byte
+ * loads are used when D % 4 == 0 and X is 16-byte aligned, else 8-byte ones),
  * D and K at most 4096; `bias` and `addend` may be NULL; `addend` (row stride
  * ldc) may be `out` itself (row stride ldo >= K): out += X . M. */
 int64_t exact_tall_gemm_table_nbytes(int64_t D, int64_t K);

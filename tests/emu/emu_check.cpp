@@ -591,6 +591,9 @@ static void check_gemm_shapes(std::mt19937& rng) {
   check_gemm(31, 604, 332, 0, rng);
   check_gemm(64, 256, 300, 4, rng);
   check_gemm(97, 48, 257, 0, rng);
+  check_gemm(67, 602, 256, 0, rng);  // D % 4 == 2: the 8-byte-load form
+  check_gemm(40, 6, 33, 2, rng);
+  check_gemm(35, 50, 70, 0, rng);
 }
 
 static const int64_t kRpShapes[][3] = {{1, 256, 32}, {31, 256, 32}, {200, 256, 32}, {130, 602, 76}, {140, 100, 25}, {129, 256, 64},

@@ -347,7 +347,7 @@ def test_pack_geometry_candidates():
 
 
 @pytest.mark.parametrize("N,D,K", [(1, 4, 1), (33, 8, 5), (70, 256, 256), (40, 128, 40), (65, 100, 47), (31, 604, 332),
-                                   (64, 256, 300), (97, 48, 257), (130, 256, 41)])
+                                   (64, 256, 300), (97, 48, 257), (130, 256, 41), (67, 602, 256), (40, 6, 33), (35, 50, 70)])
 def test_tall_gemm(N, D, K):
     """exact_tall_gemm_bf16_f32 = X . M (+ bias) (+ addend).  Small integers: every
     bf16 piece, product and partial sum is exact, so the result must be the
@@ -378,8 +378,8 @@ def test_tall_gemm_limits():
     X, M = np.zeros((8, 8), F32), np.zeros((8, 8), F32)
     assert e.emu().exact_tall_gemm_table_nbytes(0, 8) == 0 and e.emu().exact_tall_gemm_table_nbytes(8, 5000) == 0
     assert e.emu().exact_tall_gemm_table_nbytes(256, 256) == 16 * (1 + 16 * 8 * 3 * 64)
-    assert e.emu().exact_tall_gemm_bf16_f32(e.p(np.zeros((4, 6), F32)), e.p(np.zeros(1024, F32)), 4, 6, 8, None, None, 8,
-                                            e.p(np.zeros((4, 8), F32)), 8, None) == -3        # D % 4 != 0
+    assert e.emu().exact_tall_gemm_bf16_f32(e.p(np.zeros((4, 7), F32)), e.p(np.zeros(1024, F32)), 4, 7, 8, None, None, 8,
+                                            e.p(np.zeros((4, 8), F32)), 8, None) == -3        # D odd
     assert e.emu().exact_tall_gemm_bf16_f32(e.p(X), e.p(np.zeros(4096, F32)), 8, 8, 8, None, None, 8, e.p(np.zeros((8, 8), F32)), 7,
                                             None) == -3                                              # ldo < K
     assert e.emu().exact_tall_gemm_bf16_f32(None, None, 0, 8, 8, None, None, 8, None, 8, None) == 0   # N == 0: nothing to do

@@ -58,7 +58,7 @@ def test_weight_gradient_is_the_integer_product_at_benchmark_size(cuda, N, K, D,
 
 # (D, K) of the dense products x . M of the benchmark models: F.linear with M = W^T, the input gradient with M = W,
 # and the first SAGE layer's x [R | W_l^T]; plus widths that cut the 256-column slabs and the 32-column tiles unevenly
-GEMM_SHAPES = [(256, 256), (128, 256), (256, 40), (100, 256), (256, 47), (604, 332), (256, 300), (64, 1024), (1024, 64), (8, 8)]
+GEMM_SHAPES = [(256, 256), (128, 256), (256, 40), (100, 256), (256, 47), (604, 332), (256, 300), (64, 1024), (1024, 64), (8, 8), (602, 256), (50, 121)]
 
 
 @pytest.mark.parametrize("N", BIG)
