@@ -347,6 +347,7 @@ __global__ __launch_bounds__(kWave) void rp_fwd_pack_bf16_kernel(const RpPackArg
 // and written by the same lane).  The fragments of M come from
 // exact_tall_gemm_prepare_bf16, which also takes M transposed (a weight as
 // F.linear holds it).  No atomics: the result does not depend on the launch.
+constexpr int kGemmXcds = 8;       // accelerator complex dies of an MI355X, each with its own L2
 constexpr int kGemmSlabTiles = 4;  // column tiles (of 32) one launch covers
 constexpr int kGemmRowTiles = 1;   // row tiles (of 32) per wavefront in the form without LDS
 constexpr int kGemmSteps = 4;      // k-steps whose loads are issued together there
@@ -466,10 +467,18 @@ __global__ __launch_bounds__(kWave) void tall_gemm_bf16_kernel(const float* __re
 template <int VEC, int RT, int NT, int KS>
 __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float* __restrict__ X,
                                                                     const u32x4* __restrict__ table, int64_t N, int D,
-                                                                    int K, int tiles, int tile0,
+                                                                    int K, int tiles, int slabs,
                                                                     const float* __restrict__ bias, const float* addend,
                                                                     int64_t ldc, float* out, int64_t ldo) {
   HIP_DYNAMIC_SHARED(u32x4, shared_frags)  // [KS][NT][3][64]
+  // One launch covers `slabs` column slabs of NT tiles each.  Workgroups are handed to the 8 XCDs (each with its own
+  // L2) round-robin by index, so the workgroups of one row block -- one per slab -- take indices 8 apart: they run on
+  // the same XCD at about the same time and all but the first find the rows of X in that L2.  The grid is a whole
+  // number of such groups; row blocks past the last row leave here, before any barrier.
+  const int64_t in_group = blockIdx.x % (kGemmXcds * slabs);
+  const int64_t row_block = blockIdx.x / (kGemmXcds * slabs) * kGemmXcds + in_group % kGemmXcds;
+  const int tile0 = static_cast<int>(in_group / kGemmXcds) * NT;
+  if (row_block * (kBlock / kWave) * (kTile * RT) >= N) return;
   constexpr int kUnits = KS * NT * 3 * kWave;             // 16-byte units per chunk
   constexpr int kPerThread = kUnits / kBlock;             // KS * NT * 3 / 4
   static_assert(kUnits % kBlock == 0, "whole units per thread");
@@ -480,7 +489,7 @@ __global__ __launch_bounds__(kBlock) void tall_gemm_lds_bf16_kernel(const float*
   // a wavefront owns RT row tiles, so that a fragment read from LDS could serve RT products.  Measured at
   // [169343, 256] x [256, 256]: 201 us with one row tile, 287 with two, 280 with three -- the kernel lives on
   // the number of wavefronts in flight (registers per wavefront), not on fragment reads; RT = 1 is what is launched
-  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlock / kWave) + wave) * (kTile * RT);
+  const int64_t row0 = (row_block * (kBlock / kWave) + wave) * (kTile * RT);
   const u32x4* frags = table + 1;
   const float* xrow[RT];
 #pragma unroll
@@ -885,15 +894,17 @@ int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64
 #endif
   constexpr int kLdsRowTiles = EXACT_GEMM_LDS_ROW_TILES;  // row tiles per wavefront in the LDS form
   const int64_t lrows = static_cast<int64_t>(4) * kTile * kLdsRowTiles;  // four wavefronts
-  const dim3 lgrid(static_cast<unsigned>((N + lrows - 1) / lrows)), lblock(kBlock);
+  const int64_t lgroups = ((N + lrows - 1) / lrows + kGemmXcds - 1) / kGemmXcds;  // groups of 8 row blocks
+  if (lgroups * kGemmXcds * (tiles / kGemmSlabTiles + 1) > 0x7FFFFFFF) return EXACT_E_SHAPE;
+  const dim3 lblock(kBlock);
 #define EXACT_GEMM_LDS(NTV, KSV)                                                                                    \
   do {                                                                                                              \
     if (quads)                                                                                                      \
       hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<4, kLdsRowTiles, NTV, KSV>), lgrid, lblock,                     \
-                         sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, tiles, tile0, bias, addend, ldc, out, ldo); \
+                         sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, tiles, slabs, bias, addend, ldc, out, ldo); \
     else                                                                                                            \
       hipLaunchKernelGGL((tall_gemm_lds_bf16_kernel<2, kLdsRowTiles, NTV, KSV>), lgrid, lblock,                     \
-                         sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, tiles, tile0, bias, addend, ldc, out, ldo); \
+                         sizeof(u32x4) * KSV * NTV * 3 * kWave, s, X, t, N, d, kk, tiles, slabs, bias, addend, ldc, out, ldo); \
   } while (0)
 #define EXACT_GEMM_GO(NTV)                                                                                          \
   do {                                                                                                              \
@@ -905,16 +916,17 @@ int exact_tall_gemm_bf16_f32(const float* X, const void* table, int64_t N, int64
                          tile0, bias, addend, ldc, out, ldo);                                                      \
   } while (0)
   if (tiles == 2) {
-    const int tile0 = 0;
+    const int slabs = 1;
+    const dim3 lgrid(static_cast<unsigned>(lgroups * kGemmXcds));
     EXACT_GEMM_LDS(2, 4);
     return launch_status();
   }
-  for (int tile0 = 0; tile0 < tiles; tile0 += kGemmSlabTiles) {
-    const int nt = tiles - tile0 < kGemmSlabTiles ? tiles - tile0 : kGemmSlabTiles;
-    if (nt == 4) {
-      EXACT_GEMM_LDS(4, 2);
-      continue;
-    }
+  if (const int slabs = tiles / kGemmSlabTiles) {  // every full slab of four tiles in one launch
+    const dim3 lgrid(static_cast<unsigned>(lgroups * kGemmXcds * slabs));
+    EXACT_GEMM_LDS(4, 2);
+  }
+  if (const int tile0 = tiles / kGemmSlabTiles * kGemmSlabTiles; tile0 < tiles) {  // a last, narrower slab
+    const int nt = tiles - tile0;
     switch (nt) {
       case 1: EXACT_GEMM_GO(1); break;
       case 2: EXACT_GEMM_GO(2); break;
