@@ -36,22 +36,39 @@ __global__ __launch_bounds__(kBlock) void dw_zero_kernel(float* __restrict__ out
   if (i < n) out[i] = 0.f;
 }
 
+constexpr int kDwXcds = 8;   // accelerator complex dies of an MI355X, each with its own L2
+
+// Workgroup index -> (block of dW, row slab).  Every block of dW reads the same rows of dY and X over a slab, and
+// workgroups are handed to the 8 XCDs round-robin by index: the `blocks` workgroups of one slab take indices 8
+// apart, so they run on one XCD at about the same time and the rows come from HBM once and from that L2 afterwards.
+// The grid is a whole number of groups of 8 slabs; false for a slab past the last one.
+__device__ __forceinline__ bool dw_block_and_slab(int blocks, int64_t slabs, int& block, int64_t& slab) {
+  const int64_t per_group = static_cast<int64_t>(kDwXcds) * blocks;
+  const int64_t in_group = blockIdx.x % per_group;
+  block = static_cast<int>(in_group / kDwXcds);
+  slab = blockIdx.x / per_group * kDwXcds + in_group % kDwXcds;
+  return slab < slabs;
+}
+
 // WK x (4 / WK) wavefronts per workgroup along Kout x D.
 template <int MK, int MD, int WK>
 __global__ __launch_bounds__(kBlock) void linear_dw_kernel(const float* __restrict__ dY, int64_t ldy,
                                                            const float* __restrict__ X, int64_t ldx, int64_t N,
-                                                           int Kout, int D, int64_t rows_per_slab, int blocks_d,
+                                                           int Kout, int D, int64_t rows_per_slab, int blocks_d, int blocks, int64_t slabs,
                                                            float* __restrict__ out) {
   constexpr int WD = 4 / WK;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x >> 6;
   const int half = lane >> 5;
   const int l32 = lane & 31;
-  const int bk = blockIdx.x / blocks_d, bd = blockIdx.x % blocks_d;
+  int block;
+  int64_t slab;
+  if (!dw_block_and_slab(blocks, slabs, block, slab)) return;  // whole workgroup
+  const int bk = block / blocks_d, bd = block % blocks_d;
   const int k0 = (bk * WK + wave / WD) * (32 * MK);
   const int d0 = (bd * WD + wave % WD) * (32 * MD);
   if (k0 >= Kout || d0 >= D) return;  // whole wavefront: no barrier follows
-  const int64_t n_begin = static_cast<int64_t>(blockIdx.y) * rows_per_slab;
+  const int64_t n_begin = slab * rows_per_slab;
   const int64_t n_end = (n_begin + rows_per_slab < N) ? n_begin + rows_per_slab : N;
 
   int kcol[MK], dcol[MD];
@@ -132,7 +149,7 @@ __global__ __launch_bounds__(kBlock) void linear_dw_kernel(const float* __restri
 template <int MK, int MD, int WK>
 __global__ __launch_bounds__(kBlock, 2) void linear_dw_bf16_kernel(const float* __restrict__ dY, int64_t ldy,
                                                                 const float* __restrict__ X, int64_t ldx, int64_t N,
-                                                                int Kout, int D, int64_t rows_per_slab, int blocks_d,
+                                                                int Kout, int D, int64_t rows_per_slab, int blocks_d, int blocks, int64_t slabs,
                                                                 float* __restrict__ out) {
   constexpr int WD = 4 / WK;
   constexpr int64_t kRows = 16;  // rows per step
@@ -140,11 +157,14 @@ __global__ __launch_bounds__(kBlock, 2) void linear_dw_bf16_kernel(const float* 
   const int wave = threadIdx.x >> 6;
   const int half = lane >> 5;
   const int l32 = lane & 31;
-  const int bk = blockIdx.x / blocks_d, bd = blockIdx.x % blocks_d;
+  int block;
+  int64_t slab;
+  if (!dw_block_and_slab(blocks, slabs, block, slab)) return;  // whole workgroup
+  const int bk = block / blocks_d, bd = block % blocks_d;
   const int k0 = (bk * WK + wave / WD) * (32 * MK);
   const int d0 = (bd * WD + wave % WD) * (32 * MD);
   if (k0 >= Kout || d0 >= D) return;  // whole wavefront: no barrier follows
-  const int64_t n_begin = static_cast<int64_t>(blockIdx.y) * rows_per_slab;
+  const int64_t n_begin = slab * rows_per_slab;
   const int64_t n_end = (n_begin + rows_per_slab < N) ? n_begin + rows_per_slab : N;
 
   int kcol[MK], dcol[MD];
@@ -244,9 +264,9 @@ static void launch_dw(const float* dY, int64_t ldy, const float* X, int64_t ldx,
   if (rows < 512) rows = 512;
   rows = (rows + 15) / 16 * 16;  // whole batches (8 rows) resp. steps (16 rows)
   slabs = (N + rows - 1) / rows;
-  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(slabs));
-  if (BF16) hipLaunchKernelGGL((linear_dw_bf16_kernel<MK, MD, WK>), grid, dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, out);
-  else hipLaunchKernelGGL((linear_dw_kernel<MK, MD, WK>), grid, dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, out);
+  const dim3 grid(static_cast<unsigned>((slabs + kDwXcds - 1) / kDwXcds * kDwXcds * blocks));
+  if (BF16) hipLaunchKernelGGL((linear_dw_bf16_kernel<MK, MD, WK>), grid, dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, blocks, slabs, out);
+  else hipLaunchKernelGGL((linear_dw_kernel<MK, MD, WK>), grid, dim3(kBlock), 0, s, dY, ldy, X, ldx, N, Kout, D, rows, blocks_d, blocks, slabs, out);
 }
 
 template <bool BF16>
