@@ -367,6 +367,12 @@ def test_tall_gemm(N, D, K):
     assert np.array_equal(e.tall_gemm(X, M, bias=bias), (exact + bias).astype(F32))
     assert np.array_equal(e.tall_gemm(X, M, bias=bias, addend=add), (exact + bias + add).astype(F32))
     assert np.array_equal(e.tall_gemm(X, M, addend=add, in_place=True), (exact + add).astype(F32))
+    raw = np.zeros(N * D + 8, F32)                       # rows that start 8 bytes into a 16-byte line: 8-byte loads
+    first = ((8 - raw.ctypes.data % 16) % 16) // 4
+    X8 = raw[first:first + N * D].reshape(N, D); X8[:] = X
+    if D % 2 == 0:
+        assert X8.ctypes.data % 16 == 8
+        assert np.array_equal(e.tall_gemm(X8, M, bias=bias), (exact + bias).astype(F32))
     X = (rng.standard_normal((N, D)) * np.exp(rng.uniform(-4, 4, (N, 1)))).astype(F32)
     M = (rng.standard_normal((D, K)) * np.exp(rng.uniform(-4, 4, (1, K)))).astype(F32)
     want = X.astype(np.float64) @ M.astype(np.float64)

@@ -113,6 +113,24 @@ def test_tall_gemm_accuracy_and_the_framework_gemm(cuda, N, D, K):
     assert (mine / (bound + 1e-30)).max().item() <= 4 * max((theirs / (bound + 1e-30)).max().item(), 2.0 ** -24)
 
 
+def test_tall_gemm_takes_rows_aligned_to_eight_bytes(cuda):
+    """An operand that starts 8 bytes into a 16-byte line (a view into a larger
+    buffer), with a feature count that is and is not a multiple of 4: the kernel
+    reads it with 8-byte loads; integer operands, exact result."""
+    config.matrix_cores, config.tall_gemm_min_depth = "bf16", 1
+    for D, K in ((256, 256), (602, 40), (50, 300)):
+        print(f"case gemm 8-byte aligned D={D} K={K}", flush=True)
+        N = 40001
+        flat = _ints((N * D + 2,), cuda, D + K, -5, 6)
+        x = flat[2:].view(N, D)
+        assert x.data_ptr() % 16 == 8 and x.is_contiguous()
+        m = _ints((D, K), cuda, D, -5, 6)
+        with torch.no_grad():
+            got = bf.tall_matmul(x, m)
+        assert hasattr(m, "_exact_gemm_table")
+        assert torch.equal(got.double(), x.double() @ m.double())
+
+
 def test_tall_gemm_reprepares_a_changed_matrix(cuda):
     """The fragment table is remembered on the matrix and rebuilt when it changes in place (an optimiser step)."""
     config.matrix_cores = "bf16"
