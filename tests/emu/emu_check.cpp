@@ -554,16 +554,19 @@ static void check_gemm(int64_t N, int64_t D, int64_t K, int64_t pad, std::mt1993
   const int64_t tbytes = exact_tall_gemm_table_nbytes(D, K);
   CHECK(tbytes > 0 && tbytes % 16 == 0, "gemm table size");
   Buf<uint32_t> table(tbytes / 4);
-  for (int variant = 0; variant < 4; ++variant) {
+  // variant 4: the rows start 8 bytes into a 16-byte line (and still end where the allocation ends)
+  Buf<float> X8(static_cast<size_t>(N * D + 2));
+  for (int64_t i = 0; i < N * D; ++i) X8[i + 2] = X[i];
+  for (int variant = 0; variant < (D % 2 == 0 ? 5 : 4); ++variant) {
     const bool transposed = variant & 1;
     CHECK(exact_tall_gemm_prepare_bf16(transposed ? Mt.p : M.p, transposed ? ldt : ld, transposed, D, K, table.p, nullptr) == 0,
           "gemm prepare rc");
-    const bool with_bias = variant >= 1, with_add = variant >= 2, in_place = variant == 3;
+    const bool with_bias = variant >= 1, with_add = variant == 2 || variant == 3, in_place = variant == 3;
     for (int64_t i = 0; i < N * ldo; ++i) out[i] = -777.f;
     if (in_place)
       for (int64_t n = 0; n < N; ++n)
         for (int64_t c = 0; c < K; ++c) out[n * ldo + c] = add[n * ldc + c];
-    const int rc = exact_tall_gemm_bf16_f32(X.p, table.p, N, D, K, with_bias ? bias.p : nullptr,
+    const int rc = exact_tall_gemm_bf16_f32(variant == 4 ? X8.p + 2 : X.p, table.p, N, D, K, with_bias ? bias.p : nullptr,
                                             with_add ? (in_place ? out.p : add.p) : nullptr, in_place ? ldo : ldc, out.p, ldo, nullptr);
     CHECK(rc == 0, "gemm rc %d", rc);
     for (int64_t n = 0; n < N; ++n)
